@@ -7,4 +7,4 @@ Everything below the adapters runs on hand-written HIP kernels through ``libprom
 """
 from .pml import CompactSpaces, Prompt, Schema, read_file  # noqa: F401
 from .cache_engine import CacheEngine  # noqa: F401
-from .generation_engine import GenerationEngine, GenerationParameters  # noqa: F401
+from .generation_engine import BatchEngine, GenerationEngine, GenerationParameters  # noqa: F401

@@ -200,3 +200,94 @@ class GenerationEngine:
                 loop.close(len(new_ids) - 1)                 # steps of the loop that produced a token (the first came from the prefill)
             del past, loop
             gc.collect()
+
+
+class BatchEngine:
+    """Requests that step together through one model, each on a slot of the model's key arena.
+
+    The unit of work is a STEP: for every request that takes part, its next tokens (a whole prompt, a portion of one, or one
+    decoded token), run as one forward over the flat rows of all of them.  Requests join by appearing in a step, keep their
+    slot until they are ended, and a slot that was given back is handed to the next newcomer.  What a request's rows compute does
+    not depend on the rest of the step: there is no padding, and a row reads nothing but its own slot.
+
+    ``step`` is the primitive (a trace replayer calls it as it is); ``generate`` is the scheduler on top: prompts are admitted
+    while the token budget allows, prefilled together, decoded together, and leave as they finish."""
+
+    def __init__(self, lm: LanguageModel, max_tokens: Optional[int] = None):
+        model = getattr(lm, "hf_model", lm)
+        if not hasattr(model, "forward_rows"):
+            raise TypeError(f"{type(model).__name__} has no slot-addressed step (forward_rows): BatchEngine cannot drive it")
+        self.lm, self.model = lm, model
+        self.max_tokens = max_tokens
+        self.arena = None
+        self.slots = {}                       # request id -> slot
+
+    def held_tokens(self) -> int:
+        return sum(self.arena.lengths[s] for s in self.slots.values()) if self.arena is not None else 0
+
+    def _slot_for(self, rid, count: int) -> int:
+        if rid in self.slots:
+            return self.slots[rid]
+        if self.arena is None:
+            # rows as long as the budget, if one was given: then no step of this engine ever has to move the planes
+            cap = self.max_tokens if self.max_tokens else count + self.model.decode_headroom
+            self.arena = self.model.new_arena(1, max(cap, count))
+        self.slots[rid] = self.arena.alloc()
+        return self.slots[rid]
+
+    @torch.inference_mode()
+    def step(self, entries, end=()) -> torch.Tensor:
+        """``entries``: ``(request id, tokens, want)`` triples -- ``want`` the places among ``tokens`` whose logits are asked for.
+        Returns them as fp32 ``[n_wanted, vocab]`` in the order of the entries.  ``end``: requests that are finished after
+        this step; their slots are given back."""
+        entries = [(rid, list(toks), list(want)) for rid, toks, want in entries]
+        if len({rid for rid, _, _ in entries}) != len(entries):
+            raise ValueError("a request appears twice in one step")
+        logits = None
+        if entries:
+            slots = [self._slot_for(rid, len(toks)) for rid, toks, _ in entries]
+            logits = self.model.forward_rows(self.arena, slots, [t for _, t, _ in entries], [w for _, _, w in entries])
+        for rid in end:
+            if rid in self.slots:
+                self.arena.free(self.slots.pop(rid))
+        return logits
+
+    @torch.inference_mode()
+    def generate(self, prompts: List[List[int]], params: GenerationParameters) -> List[List[int]]:
+        """Token ids generated for each prompt (stop tokens included), sampled through ``params``' processor chain."""
+        processors = params.get_logits_processor()
+        out = [[] for _ in prompts]
+        waiting = list(range(len(prompts)))
+        running = []
+        budget = self.max_tokens
+        while waiting or running:
+            # admit: the waiting prompts that fit beside what the running requests may still grow to
+            admitted = []
+            if waiting:
+                used = sum(len(prompts[i]) + params.max_new_tokens for i in running)
+                for i in list(waiting):
+                    need = len(prompts[i]) + params.max_new_tokens
+                    if budget is not None and used + need > budget and (running or admitted):
+                        break
+                    admitted.append(i)
+                    waiting.remove(i)
+                    used += need
+            if admitted:
+                # (newcomers' prompts and the running requests' last tokens are different kinds of rows, yet one step takes both)
+                entries = [(i, prompts[i], [len(prompts[i]) - 1]) for i in admitted] + \
+                          [(i, [out[i][-1]], [0]) for i in running]
+                order = admitted + running
+            else:
+                entries = [(i, [out[i][-1]], [0]) for i in running]
+                order = list(running)
+            logits = self.step(entries)
+            done = []
+            for row, i in enumerate(order):
+                history = torch.as_tensor([prompts[i] + out[i]], device=logits.device) if params.repetition_penalty > 1.0 else None
+                tok = GenerationEngine._pick(processors(history, logits[row:row + 1])[0], params.greedy)
+                out[i].append(tok)
+                if tok in params.stop_token_ids or len(out[i]) >= params.max_new_tokens:
+                    done.append(i)
+            running = [i for i in order if i not in done]
+            self.step([], end=done)
+        return out

@@ -8,6 +8,9 @@ Mirrors ``promptcache/model/__init__.py`` of the reference: ``FormatConversation
 ``Falcon`` (reference :206-258) runs the same kernels through ``falcon_hip.FalconHIP`` (multi-query cache shape
 ``(L, 1, D)``) and ``Mpt`` (reference :261-288) through ``mpt_hip.MptHIP`` (ALiBi at the keys' position ids,
 ``use_full_position_ids``).
+
+``Kazolorn`` is a design of this package's own (``config.KazolornShape``): bfloat16 / float32 building-block kernels behind the
+same adapter surface.  ``load_language_model`` picks the adapter class from a checkpoint directory's ``config.json``.
 """
 from __future__ import annotations
 
@@ -19,7 +22,7 @@ from typing import Callable, List, Optional, Tuple
 import torch
 
 from ..pml import Preprocessor, PreprocessorList, escape_xml  # noqa: F401  (re-exported like the reference)
-from .config import FALCON_SHAPES, MPT_SHAPES, SHAPES, FalconShape, LlamaShape, MptShape
+from .config import FALCON_SHAPES, MPT_SHAPES, SHAPES, FalconShape, KazolornShape, LlamaShape, MptShape, architecture_of
 from .tokenizer import StandInTokenizer
 
 # HF hub ids the reference's drivers use (demo.py:27, eval.py:36, config/*.json) -> shape presets
@@ -279,3 +282,50 @@ class Mpt(LanguageModel):
     def get_cache_shape(self) -> Tuple[int, int, int]:
         c = self.hf_model.config
         return c.num_hidden_layers, c.num_attention_heads, c.head_dim
+
+
+class Kazolorn(LanguageModel):
+    """Adapter of the Kazolorn design (``config.KazolornShape``, ``kazolorn_hip.KazolornHIP``).  A checkpoint directory holds
+    ``config.json`` and ``model.safetensors``; without one, ``shape=`` plus ``random_init=True`` (or ``weights=``) gives seeded
+    random weights.  ``dtype``: ``torch.bfloat16`` (serving) or ``torch.float32`` (everything in true 32-bit)."""
+
+    def __init__(self, name: Optional[str] = None, device: str = "cuda:0", shape: Optional[KazolornShape] = None,
+                 weights=None, tokenizer=None, random_init: bool = False, seed: int = 0, dtype=torch.bfloat16, **_kwargs):
+        from .kazolorn_hip import KazolornHIP
+        from . import weights as W
+
+        if weights is not None:
+            assert shape is not None, "pass shape= together with weights="
+        elif name is not None and os.path.isdir(name):
+            shape = shape or KazolornShape.from_dir(name)
+            weights = W.load_kazolorn_safetensors(name, shape)
+        else:
+            if shape is None or not random_init:
+                raise FileNotFoundError(f"no checkpoint directory {name!r}: pass one, or shape= with random_init=True")
+            weights = W.make_kazolorn_weights(shape, seed, device=device)
+        if tokenizer is None:
+            tokenizer = StandInTokenizer(max(shape.vocab_size, 512))
+        model = KazolornHIP(shape, weights, device=device, dtype=dtype)
+        self.formatter = FormatConversation(system=("", "\n\n", ""), user=("User: ", "\n\nAssistant:"), assistant=(" ", "\n\n"))
+        super().__init__(name or shape.name, model, tokenizer, [tokenizer.eos_token_id], [])
+
+    def get_formatter(self) -> Callable[[str], str]:
+        return self.formatter
+
+    def get_cache_shape(self) -> Tuple[int, int, int]:
+        """(layers, kv heads, head size) of the FIRST layer; layers may differ (``KazolornHIP.new_arena`` knows them all)."""
+        l = self.config.layers[0]
+        return len(self.config.layers), l.kv_heads, l.dim
+
+    def encode(self, text: str) -> List[int]:
+        return [t % self.config.vocab_size for t in super().encode(text)]
+
+
+ADAPTERS = {"llama": Llama2, "falcon": Falcon, "mpt": Mpt, "kazolorn": Kazolorn}
+
+
+def load_language_model(path: str, **kwargs) -> LanguageModel:
+    """The adapter for a checkpoint directory, chosen by what its ``config.json`` says it holds."""
+    if not os.path.isdir(path):
+        raise FileNotFoundError(f"no checkpoint directory {path!r}")
+    return ADAPTERS.get(architecture_of(path), Llama2)(path, **kwargs)

@@ -186,3 +186,119 @@ SHAPES = {
     "codellama-7b": LlamaShape(vocab_size=32016, rope_theta=1e6, max_position_embeddings=16384,
                                name="codellama-7b"),
 }
+
+
+@dataclass
+class KazolornLayer:
+    """One layer of a Kazolorn stack: an attention mixer and, beside it (both read the layer's input), an optional
+    feed-forward.  ``window`` 0 = every earlier key; ``mlp_kind`` None | "dense" | "moe"."""
+    heads: int
+    kv_heads: int
+    dim: int
+    scale: float
+    window: int = 0
+    mlp_kind: object = None
+    ff: int = 0
+    experts: int = 0
+    top: int = 0
+
+
+@dataclass
+class KazolornShape:
+    """Kazolorn: decoder-only, parallel layers (mixer and feed-forward of the same input, each behind its own RMS norm and a
+    learned per-channel layer scale), a learned weighted sum of all earlier layer results in front of every layer, attention
+    without a value projection (the keys are the values) with a linear distance bias, cross-head score mixing, a sliding
+    window and a sink in the softmax denominator; dense feed-forwards use a polynomial-of-normalised-powers activation,
+    sparse ones a sigmoid top-k router whose weights scale the experts' inputs.  Every size and constant comes from
+    ``config.json`` (``from_config``); layers may differ from one another."""
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: list
+    name: str = "kazolorn"
+    initializer_range: float = 0.05
+
+    ARCHITECTURE = "Kazolorn"
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_config(cls, c: dict, name: str = "kazolorn") -> "KazolornShape":
+        if c.get("architecture") != cls.ARCHITECTURE:
+            raise ValueError(f"config.json describes {c.get('architecture')!r}, not {cls.ARCHITECTURE}")
+        layers = []
+        for i, lc in enumerate(c["layers"]):
+            if lc.get("type") != "attention":
+                raise ValueError(f"layer {i}: unknown mixer type {lc.get('type')!r}")
+            m = lc["mixer"]
+            heads, dim = int(m["heads"]), int(m["dim"])
+            kv = int(m.get("kv_heads", heads))
+            if heads % kv:
+                raise ValueError(f"layer {i}: {heads} query heads do not divide over {kv} key heads")
+            if int(m.get("vdim", dim)) != dim:
+                raise ValueError(f"layer {i}: the values are the keys, so vdim must equal dim ({m.get('vdim')} != {dim})")
+            mask = m.get("mask") or {}
+            lay = KazolornLayer(heads=heads, kv_heads=kv, dim=dim, scale=float(m["scale"]), window=int(mask.get("size") or 0))
+            mlp = lc.get("mlp")
+            if mlp:
+                kind = mlp.get("kind")
+                if kind == "dense":
+                    lay.mlp_kind, lay.ff = "dense", int(mlp["ff"])
+                elif kind == "moe":
+                    lay.mlp_kind, lay.ff = "moe", int(mlp["expert"]["ff"])
+                    lay.experts, lay.top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
+                    if not 1 <= lay.top <= lay.experts:
+                        raise ValueError(f"layer {i}: top {lay.top} of {lay.experts} experts")
+                else:
+                    raise ValueError(f"layer {i}: unknown feed-forward kind {kind!r}")
+            layers.append(lay)
+        return cls(vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), norm_eps=float(c["norm"]["eps"]), layers=layers,
+                   name=name)
+
+    @classmethod
+    def from_dir(cls, path: str) -> "KazolornShape":
+        with open(os.path.join(path, "config.json")) as f:
+            return cls.from_config(json.load(f), name=os.path.basename(os.path.normpath(path)))
+
+    def to_config(self) -> dict:
+        """The ``config.json`` form (what ``from_config`` reads)."""
+        out = []
+        for l in self.layers:
+            mixer = {"dim": l.dim, "heads": l.heads, "kv_heads": l.kv_heads, "scale": l.scale, "vdim": l.dim}
+            if l.window:
+                mixer["mask"] = {"size": l.window}
+            mlp = None
+            if l.mlp_kind == "dense":
+                mlp = {"kind": "dense", "ff": l.ff}
+            elif l.mlp_kind == "moe":
+                mlp = {"kind": "moe", "expert": {"ff": l.ff}, "router": {"experts": l.experts, "top": l.top}}
+            out.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+        return {"architecture": self.ARCHITECTURE, "layers": out, "norm": {"eps": self.norm_eps}, "vocab": self.vocab_size,
+                "width": self.hidden_size}
+
+    @classmethod
+    def uniform(cls, vocab: int, width: int, n_layers: int, heads: int, kv_heads: int, dim: int, window: int, ff: int,
+                experts: int = 0, top: int = 0, expert_ff: int = 0, dense_first: int = 1, eps: float = 1e-6,
+                name: str = "kazolorn") -> "KazolornShape":
+        """A stack of equal layers: the first ``dense_first`` with a dense feed-forward, the rest sparse (dense when
+        ``experts`` is 0)."""
+        layers = []
+        for i in range(n_layers):
+            lay = KazolornLayer(heads=heads, kv_heads=kv_heads, dim=dim, scale=dim ** -0.5, window=window)
+            if experts and i >= dense_first:
+                lay.mlp_kind, lay.ff, lay.experts, lay.top = "moe", expert_ff, experts, top
+            else:
+                lay.mlp_kind, lay.ff = "dense", ff
+            layers.append(lay)
+        return cls(vocab_size=vocab, hidden_size=width, norm_eps=eps, layers=layers, name=name)
+
+
+def architecture_of(path: str) -> str:
+    """Which model family a checkpoint directory holds: ``architecture`` (Kazolorn) or HF's ``model_type``."""
+    with open(os.path.join(path, "config.json")) as f:
+        c = json.load(f)
+    if c.get("architecture") == KazolornShape.ARCHITECTURE:
+        return "kazolorn"
+    return str(c.get("model_type", "llama"))

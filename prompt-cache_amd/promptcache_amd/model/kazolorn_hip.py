@@ -1,0 +1,299 @@
+"""Kazolorn forward pass on MI355X (``config.KazolornShape`` says what the design is).
+
+Unlike the fp16 split-plane stacks of ``llama_hip.py`` this model keeps plain row-major tensors in ONE element type --
+bfloat16 (the serving mode: matrix products on the bf16 matrix cores with fp32 accumulation) or float32 (everything in true
+32-bit) -- and an fp32 residual stream; its kernels are the building blocks of ``libpromptcache_blocks.so`` (``_blocks.py``).
+
+A step works on FLAT rows: the new tokens of all requests of the step one after another, each request appending behind the
+positions its slot of the ``SlotArena`` already holds.  No padding exists anywhere, so a request's rows see the same
+arithmetic whatever else is in the step; what a row reads from other rows is its own slot's keys and nothing else.
+
+Per layer i (x = the layer's input, X_j = earlier results, X_0 = the embedding rows):
+
+    x        = sum_j dwa_(i-1)[j] X_j              (i > 0; fused with the two norms: pcb_mix_norm)
+    h1, h2   = rms(x) g1, rms(x) g2
+    q | k    = Wqk h1 + b                          (one projection; the k part lands in the slot's cache rows)
+    a        = attention(q, cached k; values = keys, distance bias, head mixing, window, sink)      (pcb_attn_talk)
+    X_(i+1)  = x + ls1 * (Wo a + bo)               (projection epilogue)
+    X_(i+1) += ls2 * ff(h2)                        (dense: up -> polynorm -> down's epilogue;
+                                                    sparse: router -> bucket by expert -> gated units on w*h2 -> combine)
+
+and the logits are ``head . rms(sum_j dwa_last[j] X_j) g`` for the rows that were asked for.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .. import _blocks as B
+from .config import KazolornShape
+from .kv_arena import SlotArena
+from .llama_hip import CausalLMOutput
+
+ATTN_SCRATCH_FLOATS = 1 << 28          # the score band of one attention call is kept below 1 GiB (more rows: several calls)
+
+
+def distance_slopes(heads: int) -> torch.Tensor:
+    """slope_h = 2 ** (-8 (h + 1) / H), h = 0 .. H - 1, any head count."""
+    return torch.tensor([2.0 ** (-8.0 * (h + 1) / heads) for h in range(heads)], dtype=torch.float32)
+
+
+class SlotKV:
+    """``past_key_values`` of this model: the arena and the slots of the batch rows, in order."""
+
+    def __init__(self, arena: SlotArena, slots: List[int]):
+        self.arena, self.slots = arena, list(slots)
+
+    def __len__(self):
+        return len(self.arena.planes)
+
+    def __del__(self):
+        try:
+            for s in self.slots:
+                if s in self.arena._live:
+                    self.arena.free(s)
+        except Exception:
+            pass
+
+
+class KazolornHIP:
+    def __init__(self, shape: KazolornShape, weights: Dict[str, torch.Tensor], device="cuda:0", dtype=torch.bfloat16,
+                 decode_headroom: int = 256):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("Kazolorn runs in bfloat16 or float32")
+        B.load()                                   # fail loudly (or build once) before anything else
+        self.config = shape
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.decode_headroom = decode_headroom
+        self.L = len(shape.layers)
+        self.W, self.V = shape.hidden_size, shape.vocab_size
+        dev = self.device
+
+        def e(name):                               # element-type tensor (projections, biases, tables)
+            return weights[name].to(device=dev, dtype=dtype).contiguous()
+
+        def f(name):                               # fp32 tensor (gains, scales, coefficients, routers)
+            return weights[name].to(device=dev, dtype=torch.float32).contiguous()
+
+        self.embed = e("embed")
+        self.final_norm = f("final.norm")
+        self.head = e("head")
+        self.layers = []
+        for i, l in enumerate(shape.layers):
+            p = f"l{i}."
+            ent = dict(cfg=l, g1=f(p + "norm1"), ls1=f(p + "ls1"), dwa=f(p + "dwa"),
+                       wqk=torch.cat([e(p + "mix.q"), e(p + "mix.k")], dim=0).contiguous(),
+                       bqk=torch.cat([e(p + "mix.q.b"), e(p + "mix.k.b")], dim=0).contiguous(),
+                       talk=f(p + "mix.talk"), wo=e(p + "mix.o"), bo=e(p + "mix.o.b"),
+                       slopes=distance_slopes(l.heads).to(dev))
+            if ent["dwa"].numel() != i + 2:
+                raise ValueError(f"{p}dwa has {ent['dwa'].numel()} weights, layer {i} sums {i + 2} streams")
+            if l.mlp_kind:
+                ent.update(g2=f(p + "norm2"), ls2=f(p + "ls2"))
+            if l.mlp_kind == "dense":
+                ent.update(up=e(p + "mlp.up"), down=e(p + "mlp.down"), act=f(p + "mlp.act"))
+            elif l.mlp_kind == "moe":
+                ent.update(router=f(p + "mlp.router"),
+                           gate=torch.stack([e(p + f"mlp.e{j}.gate") for j in range(l.experts)]).contiguous(),
+                           up=torch.stack([e(p + f"mlp.e{j}.up") for j in range(l.experts)]).contiguous(),
+                           down=torch.stack([e(p + f"mlp.e{j}.down") for j in range(l.experts)]).contiguous())
+            self.layers.append(ent)
+        self._buf = {}
+        self.default_arena: Optional[SlotArena] = None
+
+    # ---- cache -------------------------------------------------------------------------------------------------------------
+    def new_arena(self, slots: int, cap: int) -> SlotArena:
+        return SlotArena([(l.kv_heads, l.dim) for l in self.config.layers], slots, cap, self.device, self.dtype)
+
+    def kv_bytes_per_token(self) -> int:
+        return sum(l.kv_heads * l.dim for l in self.config.layers) * (2 if self.dtype == torch.bfloat16 else 4)
+
+    # ---- scratch -----------------------------------------------------------------------------------------------------------
+    def _scratch(self, name: str, numel: int, dtype) -> torch.Tensor:
+        """A named scratch buffer of at least ``numel`` elements (grown by doubling, never shrunk)."""
+        t = self._buf.get(name)
+        if t is None or t.numel() < numel or t.dtype != dtype:
+            n = max(numel, 2 * t.numel() if t is not None and t.dtype == dtype else 0, 1024)
+            t = torch.empty(n, dtype=dtype, device=self.device)
+            self._buf[name] = t
+        return t
+
+    def _mat(self, name: str, rows: int, cols: int, dtype) -> torch.Tensor:
+        return self._scratch(name, max(rows, 1) * cols, dtype)[:max(rows, 1) * cols].view(max(rows, 1), cols)
+
+    # ---- one step ------------------------------------------------------------------------------------------------------------
+    @torch.inference_mode()
+    def forward_rows(self, arena: SlotArena, slots: Sequence[int], tokens: Sequence[Sequence[int]],
+                     want: Optional[Sequence[Sequence[int]]] = None, num_layers: Optional[int] = None,
+                     return_streams: bool = False):
+        """Append ``tokens[b]`` behind slot ``slots[b]`` for every b, and return fp32 logits ``[n_wanted, vocab]`` for the places
+        ``want[b]`` (indices into ``tokens[b]``; default: each request's last token), in request order.
+        ``return_streams``: also the layer inputs that follow each layer, fp32 ``[layers, rows, width]`` (for tests)."""
+        dev, E, f32 = self.device, self.dtype, torch.float32
+        counts = [len(t) for t in tokens]
+        if len(set(slots)) != len(slots) or len(slots) != len(tokens):
+            raise ValueError("one distinct slot per request")
+        if min(counts, default=1) < 1:
+            raise ValueError("every request of a step brings at least one token")
+        T = sum(counts)
+        if want is None:
+            want = [[c - 1] for c in counts]
+        for s, c in zip(slots, counts):
+            arena.room_for(s, c)
+        starts = [arena.lengths[s] for s in slots]
+        max_kv = max(st + c for st, c in zip(starts, counts))
+        W, V = self.W, self.V
+
+        # host-side tables of the step, one upload
+        ids = np.fromiter((t for req in tokens for t in req), dtype=np.int32, count=T)
+        if ids.size and (ids.min() < 0 or ids.max() >= V):
+            raise ValueError("token id outside the vocabulary")
+        row_slot = np.repeat(np.asarray(slots, dtype=np.int64), counts)
+        row_pos = np.concatenate([np.arange(st, st + c, dtype=np.int64) for st, c in zip(starts, counts)])
+        row0 = np.concatenate([[0], np.cumsum(counts)])
+        tiles = []
+        for b, (s, st, c) in enumerate(zip(slots, starts, counts)):
+            for q in range(0, c, 16):
+                tiles.append((s, st + q, min(16, c - q), int(row0[b]) + q))
+        tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 4)
+        want_rows = np.asarray([int(row0[b]) + int(w) for b, ws in enumerate(want) for w in ws], dtype=np.int32)
+        for b, ws in enumerate(want):
+            if any(not 0 <= int(w) < counts[b] for w in ws):
+                raise ValueError("a wanted place lies outside its request's tokens")
+        sigs = sorted({(l.kv_heads, l.dim) for l in self.config.layers})
+        offs = np.stack([row_slot * (g * arena.cap * d) + row_pos * d for g, d in sigs]) if T else np.zeros((len(sigs), 0), np.int64)
+        n32 = T + tiles.size + want_rows.size
+        blob = np.empty(n32 * 4 + offs.size * 8 + 8, dtype=np.uint8)
+        o64 = (n32 * 4 + 7) // 8 * 8
+        blob[:n32 * 4].view(np.int32)[:] = np.concatenate([ids, tiles.reshape(-1), want_rows])
+        blob[o64:o64 + offs.size * 8].view(np.int64)[:] = offs.reshape(-1)
+        dblob = torch.from_numpy(blob).to(dev)
+        d32 = dblob[:n32 * 4].view(torch.int32)
+        ids_d, tiles_d, want_d = d32[:T], d32[T:T + tiles.size], d32[T + tiles.size:]
+        offs_d = dblob[o64:o64 + offs.size * 8].view(torch.int64).view(len(sigs), T)
+
+        layers = self.layers if num_layers is None else self.layers[:num_layers]
+        L = len(layers)
+        hist = self._scratch("hist", (L + 1) * T * W, f32)[:(L + 1) * T * W].view(L + 1, T, W)
+        x = self._mat("x", T, W, f32)
+        h1, h2 = self._mat("h1", T, W, E), self._mat("h2", T, W, E)
+        streams = torch.empty((L, T, W), dtype=f32, device=dev) if return_streams else None
+        B.embed_rows(self.embed, ids_d, hist[0])
+        eps = self.config.norm_eps
+
+        for i, lw in enumerate(layers):
+            l = lw["cfg"]
+            has_ff = l.mlp_kind is not None
+            if i == 0:
+                B.mix_norm(hist, 1, None, lw["g1"], h1, lw.get("g2"), h2 if has_ff else None, eps=eps, n_rows=T)
+                base = hist[0]
+            else:
+                B.mix_norm(hist, i + 1, layers[i - 1]["dwa"], lw["g1"], h1, lw.get("g2"), h2 if has_ff else None, x_out=x,
+                           eps=eps, n_rows=T)
+                base = x
+                if streams is not None:
+                    streams[i - 1].copy_(x)
+            HD, GD = l.heads * l.dim, l.kv_heads * l.dim
+            q = self._mat("q", T, HD, E)
+            plane = arena.planes[i]
+            B.linear(h1, lw["wqk"], q, M=T, bias=lw["bqk"], split_n=HD, y2=plane, row_off2=offs_d[sigs.index((l.kv_heads, l.dim))],
+                     head_dim2=l.dim, head_stride2=arena.head_stride(i))
+            att = self._mat("att", T, HD, E)
+            self._attention(q, att, tiles, tiles_d, plane, arena, i, l, lw, max_kv)
+            B.linear(att, lw["wo"], hist[i + 1], M=T, epilogue=B.EPI_SCALE_ADD, bias=lw["bo"], base=base, col_scale=lw["ls1"])
+            if l.mlp_kind == "dense":
+                z = self._mat("z", T, l.ff, f32)
+                B.linear(h2, lw["up"], z, M=T)
+                act = self._mat("act", T, l.ff, E)
+                B.polynorm(z, lw["act"], act, eps, T)
+                B.linear(act, lw["down"], hist[i + 1], M=T, epilogue=B.EPI_SCALE_ADD, col_scale=lw["ls2"])
+            elif l.mlp_kind == "moe":
+                P = T * l.top
+                ex = self._scratch("moe_i", 3 * P + l.experts + 1, torch.int32)
+                sc = self._scratch("moe_f", 2 * P, f32)
+                expert, row_src, row_dst, goff = ex[:P], ex[P:2 * P], ex[2 * P:3 * P], ex[3 * P:3 * P + l.experts + 1]
+                weight, row_scale = sc[:P], sc[P:2 * P]
+                B.router_topk(h2, lw["router"], l.top, expert, weight, T)
+                B.moe_plan(expert, weight, P, l.top, l.experts, goff, row_src, row_dst, row_scale)
+                gact = self._mat("gact", P, l.ff, E)
+                B.linear(h2, lw["gate"], gact, M=P, epilogue=B.EPI_SILU_MUL, w2=lw["up"], row_src=row_src, row_scale=row_scale,
+                         group_off=goff, n_groups=l.experts)
+                pair = self._mat("pair", P, W, f32)
+                B.linear(gact, lw["down"], pair, M=P, row_dst=row_dst, group_off=goff, n_groups=l.experts)
+                B.moe_combine(pair, lw["ls2"], hist[i + 1], T, l.top)
+
+        n_want = int(want_rows.size)
+        logits = torch.empty((n_want, V), dtype=f32, device=dev)
+        if streams is not None:
+            B.mix_norm(hist, L + 1, layers[-1]["dwa"], None, None, x_out=x, eps=eps, n_rows=T)
+            streams[L - 1].copy_(x)
+        if n_want:
+            hn = self._mat("hn", n_want, W, E)
+            B.mix_norm(hist, L + 1, layers[-1]["dwa"], self.final_norm, hn, rows=want_d, eps=eps, n_rows=n_want)
+            B.linear(hn, self.head, logits, M=n_want)
+        for s, c in zip(slots, counts):
+            arena.lengths[s] += c
+        return (logits, streams) if return_streams else logits
+
+    def _attention(self, q, att, tiles, tiles_d, plane, arena, i, l, lw, max_kv):
+        band = B.attn_talk_band(l.window, max_kv)
+        per_tile = 16 * l.heads * band
+        n_tiles = tiles.shape[0]
+        chunk = max(1, ATTN_SCRATCH_FLOATS // per_tile)
+        if n_tiles <= chunk:
+            scratch = self._scratch("band", n_tiles * per_tile, torch.float32)
+            B.attn_talk(q, tiles_d, n_tiles, plane, arena.slot_stride(i), arena.head_stride(i), l.heads, l.kv_heads, l.dim, l.scale,
+                        l.window, max_kv, lw["slopes"], lw["talk"], True, scratch, att)
+            return
+        # too many rows for one score band: several calls, each over a run of tiles with rows counted from the run's first
+        scratch = self._scratch("band", chunk * per_tile, torch.float32)
+        for lo in range(0, n_tiles, chunk):
+            part = tiles[lo:lo + chunk].copy()
+            r0 = int(part[0, 3])
+            part[:, 3] -= r0
+            part_d = torch.from_numpy(part.reshape(-1)).to(self.device)
+            B.attn_talk(q[r0:], part_d, part.shape[0], plane, arena.slot_stride(i), arena.head_stride(i), l.heads, l.kv_heads, l.dim,
+                        l.scale, l.window, max_kv, lw["slopes"], lw["talk"], True, scratch, att[r0:])
+
+    # ---- the adapters' calling convention --------------------------------------------------------------------------------------
+    @torch.inference_mode()
+    def __call__(self, input_ids: torch.Tensor, position_ids: Optional[torch.Tensor] = None, past_key_values=None,
+                 attention_mask: Optional[torch.Tensor] = None, use_cache: bool = True, last_token_only: bool = False,
+                 num_layers: Optional[int] = None, **_unused) -> CausalLMOutput:
+        """``input_ids`` [B, q]; right padding is described by ``attention_mask`` [B, q] (1 = token).  Positions count from 0 in
+        each sequence and enter only as distances, so ``position_ids`` are not needed (they are accepted and ignored).
+        Logits come back as [B, q, vocab] (padded places hold zeros), or [B, 1, vocab] with ``last_token_only``."""
+        ids = input_ids.detach().to("cpu").reshape(input_ids.shape[0], -1)
+        Bn, q_len = ids.shape
+        if attention_mask is not None:
+            am = attention_mask.detach().to("cpu").reshape(Bn, -1)[:, -q_len:]
+            if bool((am[:, 1:] > am[:, :-1]).any()):
+                raise NotImplementedError("left / interior padding masks are not supported")
+            counts = [int(c) for c in am.sum(dim=1)]
+        else:
+            counts = [q_len] * Bn
+        if past_key_values is None:
+            arena = self.default_arena
+            if arena is None:
+                arena = self.default_arena = self.new_arena(Bn, q_len + self.decode_headroom)
+            past_key_values = SlotKV(arena, [arena.alloc() for _ in range(Bn)])
+        elif not isinstance(past_key_values, SlotKV) or len(past_key_values.slots) != Bn:
+            raise ValueError("past_key_values must be what an earlier call of this model returned, for the same batch")
+        arena, slots = past_key_values.arena, past_key_values.slots
+        toks = [ids[b, :counts[b]].tolist() for b in range(Bn)]
+        want = [[c - 1] for c in counts] if last_token_only else [list(range(c)) for c in counts]
+        flat = self.forward_rows(arena, slots, toks, want, num_layers=num_layers)
+        if last_token_only:
+            logits = flat.view(Bn, 1, self.V)
+        elif all(c == q_len for c in counts):
+            logits = flat.view(Bn, q_len, self.V)
+        else:
+            logits = torch.zeros((Bn, q_len, self.V), dtype=torch.float32, device=self.device)
+            at = 0
+            for b, c in enumerate(counts):
+                logits[b, :c] = flat[at:at + c]
+                at += c
+        return CausalLMOutput(logits=logits, past_key_values=past_key_values if use_cache else None)

@@ -277,3 +277,84 @@ def arena_from_past(past, n_layers: int, n_kv_heads: int, head_dim: int) -> Opti
         return a, S
     except Exception:
         return None
+
+
+class SlotArena:
+    """Key cache of designs whose layers may differ in head count and head size and keep ONE plane per layer (the values are the
+    keys): per layer a tensor ``[slots][kv_heads][cap][head_dim]``, plus the bookkeeping of a batch -- which slot belongs to whom
+    and how many positions it holds.  A request takes a slot (``alloc``), appends behind ``lengths[slot]`` and gives the slot
+    back (``free``); a freed slot is handed out again with length 0, its old rows are simply overwritten.
+
+    Rows are addressed by position (row j of a slot holds position j): nothing in the layout depends on how a sequence was cut
+    into steps or on which slot it sits in.  ``reserve`` grows the planes (more slots, longer rows) keeping every live row."""
+
+    def __init__(self, layer_dims, slots: int, cap: int, device, dtype=torch.bfloat16):
+        self.layer_dims = [(int(g), int(d)) for g, d in layer_dims]
+        self.device, self.dtype = torch.device(device), dtype
+        self.slots, self.cap = 0, 0
+        self.planes: List[torch.Tensor] = []
+        self.lengths: List[int] = []
+        self._free: List[int] = []
+        self._live = set()
+        self.generation = 0                   # bumped whenever the planes move (captured launches hold their addresses)
+        self.reserve(max(1, slots), max(1, cap))
+
+    # -- layout --------------------------------------------------------------------------------------------------------------
+    def slot_stride(self, layer: int) -> int:
+        g, d = self.layer_dims[layer]
+        return g * self.cap * d
+
+    def head_stride(self, layer: int) -> int:
+        return self.cap * self.layer_dims[layer][1]
+
+    def bytes_per_token(self) -> int:
+        return sum(g * d for g, d in self.layer_dims) * torch.empty(0, dtype=self.dtype).element_size()
+
+    def reserve(self, slots: int, cap: int) -> None:
+        """At least ``slots`` slots of at least ``cap`` positions each."""
+        slots, cap = max(slots, self.slots), max(cap, self.cap)
+        if slots == self.slots and cap == self.cap:
+            return
+        new = [torch.empty((slots, g, cap, d), device=self.device, dtype=self.dtype) for g, d in self.layer_dims]
+        keep = max([self.lengths[s] for s in self._live], default=0)
+        if keep:
+            for old, nw in zip(self.planes, new):
+                nw[:self.slots, :, :keep].copy_(old[:, :, :keep])
+        self._free += list(range(self.slots, slots))
+        self.lengths += [0] * (slots - self.slots)
+        self.planes, self.slots, self.cap = new, slots, cap
+        self.generation += 1
+
+    # -- slots ---------------------------------------------------------------------------------------------------------------
+    def alloc(self) -> int:
+        if not self._free:
+            self.reserve(self.slots + max(1, self.slots // 2), self.cap)
+        slot = min(self._free)                 # the lowest free slot: a batch that shrinks and refills stays compact
+        self._free.remove(slot)
+        self._live.add(slot)
+        self.lengths[slot] = 0
+        return slot
+
+    def free(self, slot: int) -> None:
+        if slot not in self._live:
+            raise KeyError(f"slot {slot} is not in use")
+        self._live.remove(slot)
+        self._free.append(slot)
+        self.lengths[slot] = 0
+
+    @property
+    def live(self) -> List[int]:
+        return sorted(self._live)
+
+    def room_for(self, slot: int, count: int) -> None:
+        """Make sure ``count`` more positions fit behind the slot's rows (grows every row by doubling)."""
+        need = self.lengths[slot] + count
+        if need > self.cap:
+            cap = self.cap
+            while cap < need:
+                cap *= 2
+            self.reserve(self.slots, cap)
+
+    def keys(self, layer: int, slot: int) -> torch.Tensor:
+        """``[kv_heads, length, head_dim]`` view of one slot's keys."""
+        return self.planes[layer][slot, :, :self.lengths[slot]]

@@ -244,3 +244,85 @@ def load_falcon_safetensors(path: str, cfg):
         for k, hf in names.items():
             out[f"l{i}.{k}"] = raw[f"transformer.h.{i}.{hf}"]
     return out
+
+
+# ---- Kazolorn ------------------------------------------------------------------------------------------------------------
+def kazolorn_weight_shapes(cfg) -> Dict[str, tuple]:
+    """Tensor names and shapes of a Kazolorn checkpoint (``model.safetensors``): ``embed``, per layer ``l{i}.norm1|norm2``,
+    ``l{i}.mix.q|k|o`` (+ ``.b`` biases) and ``l{i}.mix.talk`` [H, H], ``l{i}.mlp.up|down|act`` (dense) or
+    ``l{i}.mlp.router`` and ``l{i}.mlp.e{j}.gate|up|down`` (sparse), ``l{i}.ls1|ls2`` (layer scales), ``l{i}.dwa`` [i + 2]
+    (weights of the embedding output and every layer result up to this one), then ``final.norm`` and ``head``."""
+    W = cfg.hidden_size
+    s = {"embed": (cfg.vocab_size, W)}
+    for i, l in enumerate(cfg.layers):
+        p = f"l{i}."
+        s[p + "norm1"] = (W,)
+        s[p + "mix.q"], s[p + "mix.q.b"] = (l.heads * l.dim, W), (l.heads * l.dim,)
+        s[p + "mix.k"], s[p + "mix.k.b"] = (l.kv_heads * l.dim, W), (l.kv_heads * l.dim,)
+        s[p + "mix.talk"] = (l.heads, l.heads)
+        s[p + "mix.o"], s[p + "mix.o.b"] = (W, l.heads * l.dim), (W,)
+        s[p + "ls1"] = (W,)
+        if l.mlp_kind:
+            s[p + "norm2"], s[p + "ls2"] = (W,), (W,)
+        if l.mlp_kind == "dense":
+            s[p + "mlp.up"], s[p + "mlp.down"], s[p + "mlp.act"] = (l.ff, W), (W, l.ff), (4,)
+        elif l.mlp_kind == "moe":
+            s[p + "mlp.router"] = (l.experts, W)
+            for e in range(l.experts):
+                s[p + f"mlp.e{e}.gate"], s[p + f"mlp.e{e}.up"], s[p + f"mlp.e{e}.down"] = (l.ff, W), (l.ff, W), (W, l.ff)
+        s[p + "dwa"] = (i + 2,)
+    s["final.norm"] = (W,)
+    s["head"] = (cfg.vocab_size, W)
+    return s
+
+
+def make_kazolorn_weights(cfg, seed: int = 0, device="cpu", scale: float = 1.0):
+    """Seeded random weights (bfloat16 torch tensors).  Nothing is left at a value that would hide a dropped term: gains
+    and layer scales scatter around 1 and 0.5, biases are non-zero, the head-mixing matrix is the identity plus noise, the
+    depth weights favour the newest result without silencing the older ones, and the activation's four numbers differ."""
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    on_gpu = str(device) != "cpu"
+    gd = torch.Generator(device=device).manual_seed(seed) if on_gpu else g
+
+    def rnd(shape, big=False):
+        if big and on_gpu:
+            return torch.randn(shape, generator=gd, device=device, dtype=torch.float32)
+        return torch.randn(shape, generator=g, dtype=torch.float32).to(device)
+
+    out = {}
+    for name, shp in kazolorn_weight_shapes(cfg).items():
+        leaf = name.split(".", 1)[-1] if name.startswith("l") and name[1].isdigit() else name
+        if leaf in ("norm1", "norm2", "final.norm"):
+            w = 1.0 + 0.1 * rnd(shp)
+        elif leaf in ("ls1", "ls2"):
+            w = 0.5 + 0.1 * rnd(shp)
+        elif leaf == "dwa":
+            w = 0.15 * rnd(shp)
+            w[-1] += 1.0
+        elif leaf == "mix.talk":
+            w = torch.eye(shp[0], device=device) + 0.2 * rnd(shp)
+        elif leaf == "mlp.act":
+            w = torch.tensor([0.9, 0.35, -0.25, 0.1], device=device) + 0.05 * rnd(shp)
+        elif leaf.endswith(".b"):
+            w = 0.1 * rnd(shp)
+        elif leaf in ("embed",):
+            w = rnd(shp, big=True)
+        else:
+            w = (scale / (shp[-1] ** 0.5)) * rnd(shp, big=True)
+        out[name] = w.to(torch.bfloat16)
+    return out
+
+
+def load_kazolorn_safetensors(path: str, cfg):
+    """The tensors of ``<path>/model.safetensors`` by their own names, on the host, checked against the shapes the
+    configuration implies."""
+    raw = read_checkpoint_dir(path)
+    want = kazolorn_weight_shapes(cfg)
+    missing = [k for k in want if k not in raw]
+    if missing:
+        raise KeyError(f"{path}: tensors missing for this configuration: {missing[:6]}{' ...' if len(missing) > 6 else ''}")
+    for k, shp in want.items():
+        if tuple(raw[k].shape) != tuple(shp):
+            raise ValueError(f"{path}: {k} has shape {tuple(raw[k].shape)}, the configuration implies {tuple(shp)}")
+    return {k: raw[k] for k in want}
