@@ -672,6 +672,97 @@ def plan_only(args):
     print(json.dumps(out))
 
 
+def run_kazolorn(args):
+    """Throughput of the Kazolorn stack beside the MPT stack at equal width, heads, depth and feed-forward width.
+
+    Per size: one prompt of 2048 tokens (tokens/s of the prefill), then decoding at a context of 2048 with 1 and 8 requests
+    (tokens/s over all requests).  `equal` is Kazolorn shaped like MPT (as many key heads as query heads, no window, dense
+    feed-forward of 4 x width); `native` is the same width with grouped key heads, a 1024-token window and sparse layers.
+    Random weights, synthetic tokens, 4 layers (throughput per layer is what is compared)."""
+    import torch
+    import __graft_entry__ as ge
+    ge.build()
+    from promptcache_amd import BatchEngine
+    from promptcache_amd.model import Kazolorn, Mpt
+    from promptcache_amd.model.config import KazolornShape, MptShape
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    sizes = {"2k": dict(width=2048, heads=16, kv=4, experts=16, top=2, eff=2048),
+             "4k": dict(width=4096, heads=32, kv=8, experts=16, top=2, eff=4096)}
+    L, V, T, steps, warm = 4, 32000, 2048, max(4, min(args.steps, 20)), max(1, min(args.warmup, 3))
+    g = torch.Generator().manual_seed(0)
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    def kz_case(shape):
+        lm = Kazolorn(shape=shape, random_init=True, seed=0, device=dev)
+        m = lm.hf_model
+        prompt = torch.randint(0, V, (T,), generator=g).tolist()
+        res = {}
+
+        def prefill():
+            ar = m.new_arena(1, T)
+            m.forward_rows(ar, [ar.alloc()], [prompt])
+        for _ in range(warm):
+            prefill()
+        res["prefill_tok_s"] = round(T / timed(prefill, steps), 1)
+        for nb in (1, 8):
+            ar = m.new_arena(nb, T + 4 * (steps + warm) + 8)
+            slots = [ar.alloc() for _ in range(nb)]
+            m.forward_rows(ar, slots, [prompt] * nb)
+            step = lambda: m.forward_rows(ar, slots, [[7]] * nb)
+            for _ in range(warm):
+                step()
+            res[f"decode_b{nb}_tok_s"] = round(nb / timed(step, steps), 1)
+        del lm, m
+        torch.cuda.empty_cache()
+        return res
+
+    def mpt_case(width, heads):
+        shape = MptShape(vocab_size=V, hidden_size=width, num_hidden_layers=L, num_attention_heads=heads, name="mpt-eq")
+        lm = Mpt(shape=shape, random_init=True, seed=0, device=dev)
+        m = lm.hf_model
+        ids = torch.randint(0, V, (1, T), generator=g)
+        res = {}
+        prefill = lambda: m(input_ids=ids, use_cache=True)
+        for _ in range(warm):
+            prefill()
+        res["prefill_tok_s"] = round(T / timed(prefill, steps), 1)
+        for nb in (1, 8):
+            out = m(input_ids=ids.expand(nb, T).contiguous(), use_cache=True)
+            state = {"past": out.past_key_values, "n": T}
+
+            def step():
+                n = state["n"]
+                pos = torch.arange(n + 1).unsqueeze(0).expand(nb, n + 1)
+                o = m(input_ids=torch.full((nb, 1), 7, dtype=torch.long), position_ids=pos, past_key_values=state["past"], use_cache=True)
+                state["past"], state["n"] = o.past_key_values, n + 1
+            for _ in range(warm):
+                step()
+            res[f"decode_b{nb}_tok_s"] = round(nb / timed(step, steps), 1)
+        del lm, m
+        torch.cuda.empty_cache()
+        return res
+
+    out = {"metric": "kazolorn_throughput", "unit": "tokens/s", "dtype": "bf16 (Kazolorn) / fp16 split planes (MPT)", "data": "synthetic",
+           "layers": L, "prompt": T, "sizes": {}}
+    for key in args.kazolorn_sizes.split(","):
+        c = sizes[key]
+        w, h = c["width"], c["heads"]
+        eq = KazolornShape.uniform(V, w, L, h, h, w // h, 0, 4 * w, name=f"kazolorn-{key}-equal")
+        nat = KazolornShape.uniform(V, w, L, h, c["kv"], w // h, 1024, 4 * w, experts=c["experts"], top=c["top"], expert_ff=c["eff"],
+                                    name=f"kazolorn-{key}-native")
+        out["sizes"][key] = {"width": w, "heads": h, "mpt": mpt_case(w, h), "kazolorn_equal": kz_case(eq), "kazolorn_native": kz_case(nat)}
+        print(json.dumps({key: out["sizes"][key]}), file=sys.stderr, flush=True)
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -696,9 +787,16 @@ def main():
     ap.add_argument("--plan-link-gbs", type=float, default=153.0, help="--plan-only: one xGMI link, GB/s per direction")
     ap.add_argument("--plan-curve", default="", help="--plan-only: JSON of measured (rows per forward, seconds) points "
                                                       "(default profiles/r04_encode_rate_curve.json when present)")
+    ap.add_argument("--kazolorn", action="store_true",
+                    help="instead of the default workload: prefill / decode throughput of the Kazolorn design at layer sizes of "
+                         "real models (random weights), beside the MPT stack (the closest existing model) at equal size")
+    ap.add_argument("--kazolorn-sizes", default="2k,4k", help="--kazolorn: which sizes (2k, 4k)")
     args = ap.parse_args()
     if args.plan_only:
         plan_only(args)
+        return
+    if args.kazolorn:
+        run_kazolorn(args)
         return
 
     import torch

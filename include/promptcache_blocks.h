@@ -103,10 +103,10 @@ int pcb_linear(const pcb_linear_args* a, void* stream);
  * root; coef = {c0, c1, c2, c3} fp32 on the device; out is E. */
 int pcb_polynorm(const float* z, const float* coef, void* out, int32_t dtype, float eps, int32_t n_rows, int32_t ff, void* stream);
 
-/* Sigmoid router with top-k choice (fp32): logits = Wr h (Wr fp32 [n_experts][width], h E [n_rows][width]), score = sigmoid,
- * the `top` largest scores win (ties: the lower index).  pair p = r * top + k: expert[p], weight[p] = the score itself. */
-int pcb_router_topk(const void* h, int32_t dtype, const float* wr, int32_t n_rows, int32_t width, int32_t n_experts, int32_t top,
-                    int32_t* expert, float* weight, void* stream);
+/* Top-k choice of a sigmoid router: logits fp32 [n_rows][n_experts] (the router projection, e.g. pcb_linear with an fp32
+ * destination), score = sigmoid(logit), the `top` largest scores win (ties: the lower index).  pair p = r * top + k: expert[p],
+ * weight[p] = the score itself (not renormalised). */
+int pcb_router_topk(const float* logits, int32_t n_rows, int32_t n_experts, int32_t top, int32_t* expert, float* weight, void* stream);
 
 /* Bucket the pairs by expert: group_off[n_experts + 1], and per bucketed row its token (row_src), its pair (row_dst) and its
  * weight (row_scale).  One workgroup; n_pairs <= 1 << 20. */
@@ -146,6 +146,8 @@ typedef struct pcb_attn_talk_args {
     int64_t scratch_floats;
     void* out;
     int64_t ldo;
+    const int32_t* tiles64; /* optional: the same rows cut into tiles of up to 64 queries (same record) for the value pass */
+    int32_t n_tiles64;
 } pcb_attn_talk_args;
 int32_t pcb_attn_talk_band(int32_t window, int32_t max_kv_len);
 int pcb_attn_talk(const pcb_attn_talk_args* a, void* stream);

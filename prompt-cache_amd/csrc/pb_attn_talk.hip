@@ -17,96 +17,137 @@ struct TileRec {
     int32_t slot, q0, nq, row0;
 };
 
+// ---- 1. scores ---------------------------------------------------------------------------------------------------------------
+// Workgroup = one 16-query tile x KC keys; a wave owns 16-key subtiles of them, one after the other.  The tile's queries (all
+// heads) wait in LDS when they fit (q_lds), so the per-subtile traffic is the keys alone; a key fragment is loaded once per key
+// head and used by every query head of its group.
+constexpr int KC = 128;
+
 template <typename E, int HMAX>
-__global__ __launch_bounds__(256) void talk_scores_kernel(pcb_attn_talk_args a, int band) {
-    __shared__ float talk[HMAX * HMAX];
+__global__ __launch_bounds__(256) void talk_scores_kernel(pcb_attn_talk_args a, int band, int q_lds, int qld) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char dyn[];
+    __shared__ __attribute__((aligned(16))) float talk[HMAX * HMAX];      // [h][g], rows padded with zeros
     __shared__ float slope[HMAX];
-    const int H = a.H, D = a.head_dim, rep = H / a.Hkv;
+    const int H = a.H, D = a.head_dim, rep = H / a.Hkv, HD = H * D;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, group = lane >> 4, l15 = lane & 15;
     const TileRec t = reinterpret_cast<const TileRec*>(a.tiles)[blockIdx.x];
     const int window = a.window > 0 ? a.window : 0x3fffffff;
     const int i_last = t.q0 + t.nq - 1;
     const int j_min = t.q0 - window + 1 > 0 ? t.q0 - window + 1 : 0;
-    const int j0 = j_min + 64 * blockIdx.y + 16 * wave;          // this wave's 16 keys
-    if (j_min + 64 * (int)blockIdx.y > i_last) return;            // (uniform over the workgroup)
-    for (int e = tid; e < H * H; e += 256) talk[e] = a.talk ? a.talk[e] : ((e / H == e % H) ? 1.0f : 0.0f);
-    for (int e = tid; e < H; e += 256) slope[e] = a.slopes ? a.slopes[e] : 0.0f;
-    __syncthreads();
-    if (j0 > i_last) return;
-
+    const int j_blk = j_min + KC * blockIdx.y;
+    if (j_blk > i_last) return;                                   // (uniform over the workgroup)
     const E* Q = (const E*)a.q;
     const E* C = (const E*)a.cache + (int64_t)t.slot * a.slot_stride;
     const bool vec = sizeof(E) == 2 && D % 8 == 0 && a.ldq % 8 == 0 && a.head_stride % 8 == 0 && a.slot_stride % 8 == 0 &&
                      (((uintptr_t)Q | (uintptr_t)a.cache) % 16 == 0);
-    const int jk = j0 + l15;                                      // the key this lane loads (as a B-operand row)
-    const bool key_ok = jk <= i_last;
-    const bool q_ok = l15 < t.nq;
-
-    float s[HMAX][4];
-#pragma unroll
-    for (int h = 0; h < HMAX; ++h) {
-        if (h < H) {
-            const E* qrow = Q + (int64_t)(t.row0 + l15) * a.ldq + h * D;
-            const E* krow = C + (int64_t)(h / rep) * a.head_stride + (int64_t)jk * D;
-            f4 acc = f4{0.f, 0.f, 0.f, 0.f};
-            for (int k0 = 0; k0 < D; k0 += 32) {
-                const Frag<E> fq = load_frag(qrow + k0, group, q_ok ? D - k0 : 0, vec);
-                const Frag<E> fk = load_frag(krow + k0, group, key_ok ? D - k0 : 0, vec);
-                acc = mma(fq, fk, acc);
+    for (int e = tid; e < HMAX * HMAX; e += 256) {
+        const int h = e / HMAX, g2 = e % HMAX;
+        talk[e] = (h < H && g2 < H) ? (a.talk ? a.talk[h * H + g2] : (h == g2 ? 1.0f : 0.0f)) : 0.0f;
+    }
+    for (int e = tid; e < HMAX; e += 256) slope[e] = (e < H && a.slopes) ? a.slopes[e] : 0.0f;
+    E* Qs = reinterpret_cast<E*>(dyn);
+    if (q_lds) {
+        if (vec) {
+            const int cpr = HD / 8;
+            for (int e = tid; e < 16 * cpr; e += 256) {
+                const int r = e / cpr, c = (e % cpr) * 8;
+                u32x4 v = u32x4{0u, 0u, 0u, 0u};
+                if (r < t.nq) v = *reinterpret_cast<const u32x4*>(Q + (int64_t)(t.row0 + r) * a.ldq + c);
+                *reinterpret_cast<u32x4*>(Qs + r * qld + c) = v;
             }
-            // lane: key column l15 (j = j0 + l15), query rows 4 * group + r
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int dist = t.q0 + 4 * group + r - jk;
-                s[h][r] = acc[r] * a.scale - slope[h] * (float)dist;
+        } else {
+            for (int e = tid; e < 16 * HD; e += 256) {
+                const int r = e / HD, c = e % HD;
+                Qs[r * qld + c] = r < t.nq ? Q[(int64_t)(t.row0 + r) * a.ldq + c] : from_f32<E>(0.0f);
             }
         }
     }
+    __syncthreads();
+    const E* qrow0 = q_lds ? Qs + l15 * qld : Q + (int64_t)(t.row0 + l15) * a.ldq;
+    const bool q_ok = q_lds ? true : l15 < t.nq;
     const bool mix = a.talk != nullptr;
+    const int nsteps = (D + 31) / 32;
+
+    for (int sub = 0; sub < KC / 64; ++sub) {
+        const int j0 = j_blk + 64 * sub + 16 * wave;              // this wave's 16 keys
+        if (j0 > i_last) break;
+        const int jk = j0 + l15;                                  // the key this lane loads (as a B-operand row)
+        const bool key_ok = jk <= i_last;
+        float s[HMAX][4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int qr = 4 * group + r;
-        const int dist = t.q0 + qr - jk;
-        const bool ok = qr < t.nq && dist >= 0 && dist < window && jk >= 0;
-        if (!ok) continue;
-        float* dst = a.scratch + ((int64_t)(t.row0 + qr) * H) * band + dist;
+        for (int h = 0; h < HMAX; ++h) s[h][0] = s[h][1] = s[h][2] = s[h][3] = 0.0f;
+        for (int c = 0; c < a.Hkv; ++c) {
+            const E* krow = C + (int64_t)c * a.head_stride + (int64_t)jk * D;
+            Frag<E> fk[8];
 #pragma unroll
-        for (int h = 0; h < HMAX; ++h) {
-            if (h < H) {
-                float v = s[h][r];
-                if (mix) {
-                    v = 0.0f;
+            for (int st = 0; st < 8; ++st)
+                if (st < nsteps) fk[st] = load_frag(krow + 32 * st, group, key_ok ? D - 32 * st : 0, vec);
 #pragma unroll
-                    for (int g2 = 0; g2 < HMAX; ++g2)
-                        if (g2 < H) v += talk[h * H + g2] * s[g2][r];
+            for (int h = 0; h < HMAX; ++h) {
+                if (h / rep == c && h < H) {
+                    f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int st = 0; st < 8; ++st)
+                        if (st < nsteps) {
+                            const Frag<E> fq = load_frag(qrow0 + h * D + 32 * st, group, q_ok ? D - 32 * st : 0, vec);
+                            acc = mma(fq, fk[st], acc);
+                        }
+                    // lane: key column l15 (j = j0 + l15), query rows 4 * group + r
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) s[h][r] = acc[r] * a.scale - slope[h] * (float)(t.q0 + 4 * group + r - jk);
                 }
-                dst[(int64_t)h * band] = v;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int qr = 4 * group + r;
+            const int dist = t.q0 + qr - jk;
+            if (!(qr < t.nq && dist >= 0 && dist < window)) continue;
+            float* dst = a.scratch + ((int64_t)(t.row0 + qr) * H) * band + dist;
+#pragma unroll
+            for (int h = 0; h < HMAX; ++h) {
+                if (h < H) {
+                    float v = s[h][r];
+                    if (mix) {
+                        v = 0.0f;
+#pragma unroll
+                        for (int g4 = 0; g4 < HMAX; g4 += 4) {
+                            const f4 tw = *reinterpret_cast<const f4*>(&talk[h * HMAX + g4]);
+                            v += tw[0] * s[g4][r] + tw[1] * s[g4 + 1][r] + tw[2] * s[g4 + 2][r] + tw[3] * s[g4 + 3][r];
+                        }
+                    }
+                    dst[(int64_t)h * band] = v;
+                }
             }
         }
     }
 }
 
-template <typename E>
-__global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, int band) {
+// ---- 2. values ---------------------------------------------------------------------------------------------------------------
+// Workgroup = up to 64 consecutive queries of one sequence (a tile of the second table) x one head.  Row statistics first; then
+// per 32 keys: the rows' weights into LDS (hi + lo for bf16), the keys transposed into LDS once for all rows, and the
+// (16-row subtile, 16-column subtile) products dealt round-robin to the four waves.
+template <typename E, int NP>
+__global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, int band, const int32_t* tiles) {
     constexpr bool SPLIT = sizeof(E) == 2;           // bf16: P as hi + lo
-    constexpr int LD = 32 + 16 / sizeof(E);
+    constexpr int CE = 16 / sizeof(E), LD = 32 + CE;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    __shared__ float row_m[16], row_inv[16];
-    __shared__ __attribute__((aligned(16))) E Ph[16 * LD];
-    __shared__ __attribute__((aligned(16))) E Pl[SPLIT ? 16 * LD : 1];
+    __shared__ float row_m[64], row_inv[64];
+    __shared__ __attribute__((aligned(16))) E Ph[64 * LD];
+    __shared__ __attribute__((aligned(16))) E Pl[SPLIT ? 64 * LD : 1];
     E* Vt = reinterpret_cast<E*>(lds_raw);           // [D16][LD]: Vt[d][key]
     const int H = a.H, D = a.head_dim, rep = H / a.Hkv;
     const int D16 = (D + 15) / 16 * 16;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, group = lane >> 4, l15 = lane & 15;
-    const TileRec t = reinterpret_cast<const TileRec*>(a.tiles)[blockIdx.x];
+    const TileRec t = reinterpret_cast<const TileRec*>(tiles)[blockIdx.x];
     const int h = blockIdx.y;
     const int window = a.window > 0 ? a.window : 0x3fffffff;
     const int i_last = t.q0 + t.nq - 1;
     const int j_min = t.q0 - window + 1 > 0 ? t.q0 - window + 1 : 0;
     const float* S = a.scratch + ((int64_t)t.row0 * H + h) * band;         // row r of the tile: + r * H * band
     const int64_t s_row = (int64_t)H * band;
+    const int n_sub = (t.nq + 15) / 16, n_dt = D16 / 16, n_pairs = n_sub * n_dt;
 
-    // row statistics: wave w takes rows w, w + 4, ...
     for (int r = wave; r < t.nq; r += 4) {
         const int i = t.q0 + r;
         const int n = i + 1 < window ? i + 1 : window;
@@ -123,16 +164,15 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
     __syncthreads();
 
     const E* V = (const E*)a.cache + (int64_t)t.slot * a.slot_stride + (int64_t)(h / rep) * a.head_stride;
-    f4 acc[4];
+    const bool vec = D % CE == 0 && a.head_stride % CE == 0 && a.slot_stride % CE == 0 && ((uintptr_t)a.cache % 16 == 0);
+    f4 acc[NP];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
-    const int n_dt = D16 / 16;
+    for (int i = 0; i < NP; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
 
     for (int j0 = j_min; j0 <= i_last; j0 += 32) {
-        // weights of 16 rows x 32 keys
-        for (int e = tid; e < 16 * 32; e += 256) {
+        for (int e = tid; e < n_sub * 16 * 32; e += 256) {
             const int r = e >> 5, kk = e & 31;
-            const int j = j0 + kk, dist = t.q0 + r - j;
+            const int dist = t.q0 + r - (j0 + kk);
             float p = 0.0f;
             if (r < t.nq && dist >= 0 && dist < window) p = expf(S[r * s_row + dist] - row_m[r]) * row_inv[r];
             if (SPLIT) {
@@ -143,59 +183,102 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
                 Ph[r * LD + kk] = from_f32<E>(p);
             }
         }
-        // the keys as values, transposed: Vt[d][kk]
-        for (int e = tid; e < 32 * D16; e += 256) {
-            const int kk = e / D16, d = e % D16;
-            const int j = j0 + kk;
-            Vt[d * LD + kk] = (j <= i_last && d < D) ? V[(int64_t)j * D + d] : from_f32<E>(0.0f);
+        if (vec) {
+            const int cpk = D / CE;                   // 16-byte chunks per key
+            for (int e = tid; e < 32 * cpk; e += 256) {
+                const int kk = e & 31, c = (e >> 5) * CE;
+                const int j = j0 + kk;
+                __attribute__((aligned(16))) E tmp[CE];
+                if (j <= i_last)
+                    *reinterpret_cast<u32x4*>(tmp) = *reinterpret_cast<const u32x4*>(V + (int64_t)j * D + c);
+                else
+                    *reinterpret_cast<u32x4*>(tmp) = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int i = 0; i < CE; ++i) Vt[(c + i) * LD + kk] = tmp[i];
+            }
+            for (int e = tid; e < 32 * (D16 - D); e += 256) Vt[(D + e / 32) * LD + (e & 31)] = from_f32<E>(0.0f);
+        } else {
+            for (int e = tid; e < 32 * D16; e += 256) {
+                const int kk = e / D16, d = e % D16;
+                const int j = j0 + kk;
+                Vt[d * LD + kk] = (j <= i_last && d < D) ? V[(int64_t)j * D + d] : from_f32<E>(0.0f);
+            }
         }
         __syncthreads();
-        const Frag<E> ph = load_frag(&Ph[l15 * LD], group, 32, true);
-        Frag<E> pl;
-        if (SPLIT) pl = load_frag(&Pl[l15 * LD], group, 32, true);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int dt = wave + 4 * i;
-            if (dt < n_dt) {
+        for (int i = 0; i < NP; ++i) {
+            const int p = wave + 4 * i;
+            if (p < n_pairs) {
+                const int sub = p % n_sub, dt = p / n_sub;
+                const Frag<E> ph = load_frag(&Ph[(sub * 16 + l15) * LD], group, 32, true);
                 const Frag<E> fv = load_frag(&Vt[(dt * 16 + l15) * LD], group, 32, true);
                 acc[i] = mma(ph, fv, acc[i]);
-                if (SPLIT) acc[i] = mma(pl, fv, acc[i]);
+                if (SPLIT) {
+                    const Frag<E> pl = load_frag(&Pl[(sub * 16 + l15) * LD], group, 32, true);
+                    acc[i] = mma(pl, fv, acc[i]);
+                }
             }
         }
         __syncthreads();
     }
     E* O = (E*)a.out;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int d = (wave + 4 * i) * 16 + l15;
-        if (wave + 4 * i < n_dt && d < D) {
+    for (int i = 0; i < NP; ++i) {
+        const int p = wave + 4 * i;
+        if (p < n_pairs) {
+            const int sub = p % n_sub, d = (p / n_sub) * 16 + l15;
+            if (d < D) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int qr = 4 * group + r;
-                if (qr < t.nq) O[(int64_t)(t.row0 + qr) * a.ldo + h * D + d] = from_f32<E>(acc[i][r]);
+                for (int r = 0; r < 4; ++r) {
+                    const int qr = sub * 16 + 4 * group + r;
+                    if (qr < t.nq) O[(int64_t)(t.row0 + qr) * a.ldo + h * D + d] = from_f32<E>(acc[i][r]);
+                }
             }
         }
     }
 }
 
+template <typename E, int HMAX>
+void launch_scores(const pcb_attn_talk_args& a, int band, hipStream_t stream) {
+    // the tile's queries wait in LDS when 16 rows of all heads fit beside the kernel's own tables (160 KiB per workgroup)
+    const int ce = 16 / (int)sizeof(E);
+    const int qld = a.H * a.head_dim + ce;
+    const size_t q_bytes = (size_t)16 * qld * sizeof(E);
+    const bool aligned = (a.H * a.head_dim) % ce == 0;
+    const int q_lds = aligned && q_bytes + sizeof(float) * (HMAX * HMAX + HMAX) <= 150 * 1024;
+    auto kern = talk_scores_kernel<E, HMAX>;
+    static bool raised = false;
+    if (q_lds && q_bytes > 48 * 1024 && !raised) {
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        raised = true;
+    }
+    const dim3 grid(a.n_tiles, pcb_ceil_div(band + 15, KC));
+    hipLaunchKernelGGL(kern, grid, dim3(256), q_lds ? q_bytes : 0, stream, a, band, q_lds, qld);
+}
+
 template <typename E>
 int run(const pcb_attn_talk_args& a, int band, hipStream_t stream) {
     const int H = a.H;
-    const int key_blocks = pcb_ceil_div(band + 15, 64);
-    const dim3 g1(a.n_tiles, key_blocks);
     if (H <= 4)
-        hipLaunchKernelGGL((talk_scores_kernel<E, 4>), g1, dim3(256), 0, stream, a, band);
+        launch_scores<E, 4>(a, band, stream);
     else if (H <= 8)
-        hipLaunchKernelGGL((talk_scores_kernel<E, 8>), g1, dim3(256), 0, stream, a, band);
+        launch_scores<E, 8>(a, band, stream);
     else if (H <= 16)
-        hipLaunchKernelGGL((talk_scores_kernel<E, 16>), g1, dim3(256), 0, stream, a, band);
+        launch_scores<E, 16>(a, band, stream);
     else
-        hipLaunchKernelGGL((talk_scores_kernel<E, 32>), g1, dim3(256), 0, stream, a, band);
+        launch_scores<E, 32>(a, band, stream);
     int rc = pcb_check_launch("talk_scores_kernel");
     if (rc != PCB_OK) return rc;
     const int D16 = (a.head_dim + 15) / 16 * 16;
     const size_t lds = (size_t)D16 * (32 + 16 / sizeof(E)) * sizeof(E);
-    hipLaunchKernelGGL((talk_values_kernel<E>), dim3(a.n_tiles, H), dim3(256), lds, stream, a, band);
+    const int32_t* tiles = a.tiles64 ? a.tiles64 : a.tiles;
+    const dim3 grid(a.tiles64 ? a.n_tiles64 : a.n_tiles, H);
+    if (D16 <= 64)
+        hipLaunchKernelGGL((talk_values_kernel<E, 4>), grid, dim3(256), lds, stream, a, band, tiles);
+    else if (D16 <= 128)
+        hipLaunchKernelGGL((talk_values_kernel<E, 8>), grid, dim3(256), lds, stream, a, band, tiles);
+    else
+        hipLaunchKernelGGL((talk_values_kernel<E, 16>), grid, dim3(256), lds, stream, a, band, tiles);
     return pcb_check_launch("talk_values_kernel");
 }
 
@@ -214,6 +297,7 @@ PCB_EXPORT int pcb_attn_talk(const pcb_attn_talk_args* a, void* stream) {
     PCB_REQUIRE(a->n_tiles >= 0 && a->max_kv_len > 0, PCB_ERR_ARG, "pcb_attn_talk: bad sizes");
     if (a->n_tiles == 0) return PCB_OK;
     PCB_REQUIRE(a->q && a->tiles && a->cache && a->scratch && a->out, PCB_ERR_ARG, "pcb_attn_talk: null pointer");
+    PCB_REQUIRE(!a->tiles64 || a->n_tiles64 > 0, PCB_ERR_ARG, "pcb_attn_talk: the second tile table is empty");
     PCB_REQUIRE(a->ldq >= (int64_t)a->H * a->head_dim && a->ldo >= (int64_t)a->H * a->head_dim, PCB_ERR_ARG,
                 "pcb_attn_talk: row strides shorter than heads * head_dim");
     const int band = pcb_attn_talk_band(a->window, a->max_kv_len);

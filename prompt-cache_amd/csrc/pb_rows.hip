@@ -102,26 +102,18 @@ __global__ __launch_bounds__(256) void polynorm_kernel(const float* __restrict__
     }
 }
 
-// one wave per row: lane-strided dot products, scores in LDS, `top` rounds of a wave-wide arg-max
-template <typename E>
-__global__ __launch_bounds__(256) void router_topk_kernel(const E* __restrict__ h, const float* __restrict__ wr, int n_rows, int width,
-                                                          int n_experts, int top, int32_t* __restrict__ expert,
-                                                          float* __restrict__ weight) {
+// one wave per row of router logits: sigmoid scores in LDS, `top` rounds of a wave-wide arg-max
+__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits, int n_rows, int n_experts, int top,
+                                                          int32_t* __restrict__ expert, float* __restrict__ weight) {
     extern __shared__ float sc[];          // [4][n_experts]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = blockIdx.x * 4 + wave;
     if (r >= n_rows) return;
     float* s = sc + wave * n_experts;
-    const E* hr = h + (int64_t)r * width;
-    for (int e = 0; e < n_experts; ++e) {
-        const float* w = wr + (int64_t)e * width;
-        float acc = 0.0f;
-        for (int c = lane; c < width; c += 64) acc += w[c] * to_f32(hr[c]);
-        acc = wave_sum(acc);
-        if (lane == 0) s[e] = 1.0f / (1.0f + expf(-acc));
-    }
+    for (int e = lane; e < n_experts; e += 64) s[e] = 1.0f / (1.0f + expf(-logits[(int64_t)r * n_experts + e]));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     for (int k = 0; k < top; ++k) {
         float best = -1.0f;
         int bi = 0x7fffffff;
@@ -140,8 +132,9 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const E* __restrict__ 
             weight[(int64_t)r * top + k] = best;
             s[bi] = -2.0f;
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 }
 
@@ -229,20 +222,14 @@ PCB_EXPORT int pcb_polynorm(const float* z, const float* coef, void* out, int32_
     return pcb_check_launch("polynorm_kernel");
 }
 
-PCB_EXPORT int pcb_router_topk(const void* h, int32_t dtype, const float* wr, int32_t n_rows, int32_t width, int32_t n_experts,
-                               int32_t top, int32_t* expert, float* weight, void* stream) {
-    PCB_REQUIRE(PCB_DTYPE_OK(dtype) && n_rows >= 0 && width > 0 && n_experts > 0 && n_experts <= 2048 && top > 0 && top <= n_experts,
-                PCB_ERR_ARG, "pcb_router_topk: bad sizes (1 <= top <= n_experts <= 2048)");
+PCB_EXPORT int pcb_router_topk(const float* logits, int32_t n_rows, int32_t n_experts, int32_t top, int32_t* expert, float* weight,
+                               void* stream) {
+    PCB_REQUIRE(n_rows >= 0 && n_experts > 0 && n_experts <= 2048 && top > 0 && top <= n_experts, PCB_ERR_ARG,
+                "pcb_router_topk: bad sizes (1 <= top <= n_experts <= 2048)");
     if (n_rows == 0) return PCB_OK;
-    PCB_REQUIRE(h && wr && expert && weight, PCB_ERR_ARG, "pcb_router_topk: null pointer");
-    const size_t lds = (size_t)4 * n_experts * sizeof(float);
-    const dim3 grid(pcb_ceil_div(n_rows, 4));
-    if (dtype == PCB_BF16)
-        hipLaunchKernelGGL(router_topk_kernel<bf16_t>, grid, dim3(256), lds, (hipStream_t)stream, (const bf16_t*)h, wr, n_rows, width,
-                           n_experts, top, expert, weight);
-    else
-        hipLaunchKernelGGL(router_topk_kernel<float>, grid, dim3(256), lds, (hipStream_t)stream, (const float*)h, wr, n_rows, width,
-                           n_experts, top, expert, weight);
+    PCB_REQUIRE(logits && expert && weight, PCB_ERR_ARG, "pcb_router_topk: null pointer");
+    hipLaunchKernelGGL(router_topk_kernel, dim3(pcb_ceil_div(n_rows, 4)), dim3(256), (size_t)4 * n_experts * sizeof(float),
+                       (hipStream_t)stream, logits, n_rows, n_experts, top, expert, weight);
     return pcb_check_launch("router_topk_kernel");
 }
 

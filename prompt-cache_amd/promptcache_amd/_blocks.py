@@ -46,7 +46,8 @@ class AttnTalkArgs(C.Structure):
                 ("cache", _vp), ("slot_stride", _i64), ("head_stride", _i64),
                 ("H", _i32), ("Hkv", _i32), ("head_dim", _i32), ("scale", _f32), ("window", _i32), ("max_kv_len", _i32),
                 ("slopes", _vp), ("talk", _vp), ("sink", _i32),
-                ("scratch", _vp), ("scratch_floats", _i64), ("out", _vp), ("ldo", _i64)]
+                ("scratch", _vp), ("scratch_floats", _i64), ("out", _vp), ("ldo", _i64),
+                ("tiles64", _vp), ("n_tiles64", _i32)]
 
 
 # name -> (restype, argtypes); mirrors include/promptcache_blocks.h one to one
@@ -57,7 +58,7 @@ SIGNATURES = {
     "pcb_mix_norm": (C.c_int, [C.POINTER(MixNormArgs), _vp]),
     "pcb_linear": (C.c_int, [C.POINTER(LinearArgs), _vp]),
     "pcb_polynorm": (C.c_int, [_vp, _vp, _vp, _i32, _f32, _i32, _i32, _vp]),
-    "pcb_router_topk": (C.c_int, [_vp, _i32, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "pcb_router_topk": (C.c_int, [_vp, _i32, _i32, _i32, _vp, _vp, _vp]),
     "pcb_moe_plan": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "pcb_moe_combine": (C.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "pcb_attn_talk_band": (C.c_int32, [_i32, _i32]),
@@ -201,13 +202,12 @@ def polynorm(z: torch.Tensor, coef: torch.Tensor, out: torch.Tensor, eps: float,
     check(load().pcb_polynorm(_p(z), _p(coef), _p(out), _code(out), float(eps), n_rows, ff, _stream()), "pcb_polynorm")
 
 
-def router_topk(h: torch.Tensor, wr: torch.Tensor, top: int, expert: torch.Tensor, weight: torch.Tensor, n_rows: int) -> None:
-    _want(wr, torch.float32, "router_topk wr"); _want(expert, torch.int32, "router_topk expert")
+def router_topk(logits: torch.Tensor, top: int, expert: torch.Tensor, weight: torch.Tensor, n_rows: int) -> None:
+    _want(logits, torch.float32, "router_topk logits"); _want(expert, torch.int32, "router_topk expert")
     _want(weight, torch.float32, "router_topk weight")
-    E, W = wr.shape
-    assert h.is_contiguous() and h.shape[-1] == W and h.shape[0] >= n_rows and expert.numel() >= n_rows * top and \
-        weight.numel() >= n_rows * top
-    check(load().pcb_router_topk(_p(h), _code(h), _p(wr), n_rows, W, E, top, _p(expert), _p(weight), _stream()), "pcb_router_topk")
+    E = logits.shape[-1]
+    assert logits.shape[0] >= n_rows and expert.numel() >= n_rows * top and weight.numel() >= n_rows * top
+    check(load().pcb_router_topk(_p(logits), n_rows, E, top, _p(expert), _p(weight), _stream()), "pcb_router_topk")
 
 
 def moe_plan(expert: torch.Tensor, weight: torch.Tensor, n_pairs: int, top: int, n_experts: int, group_off: torch.Tensor,
@@ -234,7 +234,7 @@ def attn_talk_band(window: int, max_kv_len: int) -> int:
 
 def attn_talk(q: torch.Tensor, tiles: torch.Tensor, n_tiles: int, cache: torch.Tensor, slot_stride: int, head_stride: int,
               H: int, Hkv: int, head_dim: int, scale: float, window: int, max_kv_len: int, slopes, talk, sink: bool,
-              scratch: torch.Tensor, out: torch.Tensor) -> None:
+              scratch: torch.Tensor, out: torch.Tensor, tiles64: Optional[torch.Tensor] = None, n_tiles64: int = 0) -> None:
     _want(tiles, torch.int32, "attn_talk tiles"); _want(scratch, torch.float32, "attn_talk scratch")
     assert q.dtype == cache.dtype == out.dtype and q.is_contiguous() and out.is_contiguous() and cache.is_cuda
     assert tiles.numel() >= 4 * n_tiles and q.shape[-1] == H * head_dim and out.shape[-1] == H * head_dim
@@ -245,5 +245,8 @@ def attn_talk(q: torch.Tensor, tiles: torch.Tensor, n_tiles: int, cache: torch.T
         _want(talk, torch.float32, "attn_talk talk"); assert talk.numel() == H * H
     a = AttnTalkArgs(C.sizeof(AttnTalkArgs), _code(q), _p(q), q.shape[-1], _p(tiles), n_tiles, _p(cache), slot_stride,
                      head_stride, H, Hkv, head_dim, float(scale), int(window), int(max_kv_len), _p(slopes), _p(talk), int(sink),
-                     _p(scratch), scratch.numel(), _p(out), out.shape[-1])
+                     _p(scratch), scratch.numel(), _p(out), out.shape[-1], _p(tiles64), n_tiles64 if tiles64 is not None else 0)
+    if tiles64 is not None:
+        _want(tiles64, torch.int32, "attn_talk tiles64")
+        assert tiles64.numel() >= 4 * n_tiles64 > 0
     check(load().pcb_attn_talk(C.byref(a), _stream()), "pcb_attn_talk")

@@ -96,7 +96,7 @@ class KazolornHIP:
             if l.mlp_kind == "dense":
                 ent.update(up=e(p + "mlp.up"), down=e(p + "mlp.down"), act=f(p + "mlp.act"))
             elif l.mlp_kind == "moe":
-                ent.update(router=f(p + "mlp.router"),
+                ent.update(router=e(p + "mlp.router"),
                            gate=torch.stack([e(p + f"mlp.e{j}.gate") for j in range(l.experts)]).contiguous(),
                            up=torch.stack([e(p + f"mlp.e{j}.up") for j in range(l.experts)]).contiguous(),
                            down=torch.stack([e(p + f"mlp.e{j}.down") for j in range(l.experts)]).contiguous())
@@ -159,20 +159,23 @@ class KazolornHIP:
             for q in range(0, c, 16):
                 tiles.append((s, st + q, min(16, c - q), int(row0[b]) + q))
         tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 4)
+        tiles64 = np.asarray([(s, st + q, min(64, c - q), int(row0[b]) + q) for b, (s, st, c) in enumerate(zip(slots, starts, counts))
+                              for q in range(0, c, 64)], dtype=np.int32).reshape(-1, 4)
         want_rows = np.asarray([int(row0[b]) + int(w) for b, ws in enumerate(want) for w in ws], dtype=np.int32)
         for b, ws in enumerate(want):
             if any(not 0 <= int(w) < counts[b] for w in ws):
                 raise ValueError("a wanted place lies outside its request's tokens")
         sigs = sorted({(l.kv_heads, l.dim) for l in self.config.layers})
         offs = np.stack([row_slot * (g * arena.cap * d) + row_pos * d for g, d in sigs]) if T else np.zeros((len(sigs), 0), np.int64)
-        n32 = T + tiles.size + want_rows.size
+        n32 = T + tiles.size + want_rows.size + tiles64.size
         blob = np.empty(n32 * 4 + offs.size * 8 + 8, dtype=np.uint8)
         o64 = (n32 * 4 + 7) // 8 * 8
-        blob[:n32 * 4].view(np.int32)[:] = np.concatenate([ids, tiles.reshape(-1), want_rows])
+        blob[:n32 * 4].view(np.int32)[:] = np.concatenate([ids, tiles.reshape(-1), want_rows, tiles64.reshape(-1)])
         blob[o64:o64 + offs.size * 8].view(np.int64)[:] = offs.reshape(-1)
         dblob = torch.from_numpy(blob).to(dev)
         d32 = dblob[:n32 * 4].view(torch.int32)
-        ids_d, tiles_d, want_d = d32[:T], d32[T:T + tiles.size], d32[T + tiles.size:]
+        ids_d, tiles_d, want_d = d32[:T], d32[T:T + tiles.size], d32[T + tiles.size:T + tiles.size + want_rows.size]
+        tiles64_d = d32[T + tiles.size + want_rows.size:]
         offs_d = dblob[o64:o64 + offs.size * 8].view(torch.int64).view(len(sigs), T)
 
         layers = self.layers if num_layers is None else self.layers[:num_layers]
@@ -202,7 +205,7 @@ class KazolornHIP:
             B.linear(h1, lw["wqk"], q, M=T, bias=lw["bqk"], split_n=HD, y2=plane, row_off2=offs_d[sigs.index((l.kv_heads, l.dim))],
                      head_dim2=l.dim, head_stride2=arena.head_stride(i))
             att = self._mat("att", T, HD, E)
-            self._attention(q, att, tiles, tiles_d, plane, arena, i, l, lw, max_kv)
+            self._attention(q, att, tiles, tiles_d, tiles64_d, tiles64.shape[0], plane, arena, i, l, lw, max_kv)
             B.linear(att, lw["wo"], hist[i + 1], M=T, epilogue=B.EPI_SCALE_ADD, bias=lw["bo"], base=base, col_scale=lw["ls1"])
             if l.mlp_kind == "dense":
                 z = self._mat("z", T, l.ff, f32)
@@ -216,7 +219,9 @@ class KazolornHIP:
                 sc = self._scratch("moe_f", 2 * P, f32)
                 expert, row_src, row_dst, goff = ex[:P], ex[P:2 * P], ex[2 * P:3 * P], ex[3 * P:3 * P + l.experts + 1]
                 weight, row_scale = sc[:P], sc[P:2 * P]
-                B.router_topk(h2, lw["router"], l.top, expert, weight, T)
+                rl = self._mat("router", T, l.experts, f32)
+                B.linear(h2, lw["router"], rl, M=T)                  # fp32 accumulation of exact products: 32-bit logits
+                B.router_topk(rl, l.top, expert, weight, T)
                 B.moe_plan(expert, weight, P, l.top, l.experts, goff, row_src, row_dst, row_scale)
                 gact = self._mat("gact", P, l.ff, E)
                 B.linear(h2, lw["gate"], gact, M=P, epilogue=B.EPI_SILU_MUL, w2=lw["up"], row_src=row_src, row_scale=row_scale,
@@ -238,7 +243,7 @@ class KazolornHIP:
             arena.lengths[s] += c
         return (logits, streams) if return_streams else logits
 
-    def _attention(self, q, att, tiles, tiles_d, plane, arena, i, l, lw, max_kv):
+    def _attention(self, q, att, tiles, tiles_d, tiles64_d, n64, plane, arena, i, l, lw, max_kv):
         band = B.attn_talk_band(l.window, max_kv)
         per_tile = 16 * l.heads * band
         n_tiles = tiles.shape[0]
@@ -246,7 +251,7 @@ class KazolornHIP:
         if n_tiles <= chunk:
             scratch = self._scratch("band", n_tiles * per_tile, torch.float32)
             B.attn_talk(q, tiles_d, n_tiles, plane, arena.slot_stride(i), arena.head_stride(i), l.heads, l.kv_heads, l.dim, l.scale,
-                        l.window, max_kv, lw["slopes"], lw["talk"], True, scratch, att)
+                        l.window, max_kv, lw["slopes"], lw["talk"], True, scratch, att, tiles64=tiles64_d, n_tiles64=n64)
             return
         # too many rows for one score band: several calls, each over a run of tiles with rows counted from the run's first
         scratch = self._scratch("band", chunk * per_tile, torch.float32)

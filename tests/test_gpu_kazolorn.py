@@ -203,10 +203,12 @@ def test_polynorm(dtype):
 @pytest.mark.parametrize("E,top", [(5, 2), (1, 1), (70, 3), (12, 12)])
 def test_router_and_plan(dtype, E, top):
     T, Wd = 23, 44
-    h, wr = rnd(T, Wd, dtype=dtype, seed=1), rnd(E, Wd, seed=2, scale=0.4)
+    h, wr = rnd(T, Wd, dtype=dtype, seed=1), rnd(E, Wd, dtype=dtype, seed=2, scale=0.4)
     ex = torch.empty(T * top, dtype=torch.int32, device=DEV)
     wt = torch.empty(T * top, dtype=torch.float32, device=DEV)
-    B().router_topk(h, wr, top, ex, wt, T)
+    logits = torch.empty((T, E), dtype=torch.float32, device=DEV)
+    B().linear(h, wr, logits, M=T)
+    B().router_topk(logits, top, ex, wt, T)
     idx, val = O.route(h.to(F64).cpu(), wr.to(F64).cpu(), top)
     assert torch.equal(ex.view(T, top).cpu().long(), idx)
     assert rel(wt.view(T, top), val) < 1e-5
