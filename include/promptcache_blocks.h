@@ -123,8 +123,9 @@ int pcb_moe_combine(const float* pair_out, const float* col_scale, float* y, int
  *   - sink: one more term exp(0) in the softmax denominator that carries no value
  * Queries are flat rows; tile t = {slot, first query position, query rows (<= 16), first flat row} (int32 x 4, device).  The
  * cache holds key j of kv head g of slot s at cache + s * slot_stride + g * head_stride + j * head_dim and must already contain
- * the queries' own keys.  Query head h reads kv head h / (H / Hkv).  scratch: fp32 [n_rows_padded][H][band] with
- * band = pcb_attn_talk_band(window, max_kv_len); out is E [rows][ldo], head h at column h * head_dim. */
+ * the queries' own keys.  Query head h reads kv head h / (H / Hkv).  scratch: fp32 [n_tiles * 16][H][band] with
+ * band = pcb_attn_talk_band(window, max_kv_len) (the distances a row can see, padded); out is E [rows][ldo], head h at column
+ * h * head_dim. */
 typedef struct pcb_attn_talk_args {
     uint32_t struct_bytes;
     int32_t dtype;

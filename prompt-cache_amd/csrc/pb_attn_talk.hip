@@ -252,7 +252,7 @@ void launch_scores(const pcb_attn_talk_args& a, int band, hipStream_t stream) {
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
         raised = true;
     }
-    const dim3 grid(a.n_tiles, pcb_ceil_div(band + 15, KC));
+    const dim3 grid(a.n_tiles, pcb_ceil_div(band, KC));
     hipLaunchKernelGGL(kern, grid, dim3(256), q_lds ? q_bytes : 0, stream, a, band, q_lds, qld);
 }
 
@@ -285,8 +285,10 @@ int run(const pcb_attn_talk_args& a, int band, hipStream_t stream) {
 }  // namespace
 
 PCB_EXPORT int32_t pcb_attn_talk_band(int32_t window, int32_t max_kv_len) {
+    // rounded up to 16 floats plus 16 more: consecutive heads and rows of the band must not sit a power of two apart (their
+    // stores would crowd into a few memory channels)
     const int b = (window > 0 && window < max_kv_len) ? window : max_kv_len;
-    return b < 1 ? 1 : b;
+    return ((b < 1 ? 1 : b) + 15) / 16 * 16 + 16;
 }
 
 PCB_EXPORT int pcb_attn_talk(const pcb_attn_talk_args* a, void* stream) {

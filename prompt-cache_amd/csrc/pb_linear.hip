@@ -43,6 +43,30 @@ __device__ __forceinline__ u32x4 load_chunk(const E* p, int k, int K, bool vec, 
     return c;
 }
 
+// one result element through the epilogue (see pcb_linear_args)
+template <typename E, int EPI>
+__device__ __forceinline__ void emit(const pcb_linear_args& a, int m, int n, float acc, float acc2, float bv, float cs) {
+    float v = acc + bv;
+    if (EPI == PCB_EPI_SILU_MUL) v = acc / (1.0f + expf(-acc)) * acc2;
+    if (EPI == PCB_EPI_SCALE_ADD) {
+        float* y = (float*)a.y + (int64_t)m * a.ldy + n;
+        const float b0 = a.base ? a.base[(int64_t)m * a.ldbase + n] : *y;
+        *y = b0 + cs * v;
+        return;
+    }
+    if (a.split_n > 0 && n >= a.split_n) {
+        const int c = n - a.split_n;
+        E* y = (E*)a.y2 + a.row_off2[m] + (int64_t)(c / a.head_dim2) * a.head_stride2 + c % a.head_dim2;
+        *y = from_f32<E>(v);
+        return;
+    }
+    const int64_t at = (int64_t)(a.row_dst ? a.row_dst[m] : m) * a.ldy + n;
+    if (a.out_f32)
+        ((float*)a.y)[at] = v;
+    else
+        ((E*)a.y)[at] = from_f32<E>(v);
+}
+
 template <typename E, int EPI, int TM, int TN>
 __global__ __launch_bounds__(256) void linear_kernel(pcb_linear_args a) {
     constexpr bool TWO = EPI == PCB_EPI_SILU_MUL;
@@ -171,30 +195,100 @@ __global__ __launch_bounds__(256) void linear_kernel(pcb_linear_args a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = m_lo + (wm * TM + i) * 16 + 4 * group + r;
-                if (m >= m_hi) continue;
-                float v = acc[i][j][r] + bv;
-                if (EPI == PCB_EPI_SILU_MUL) {
-                    const float gte = acc[i][j][r];
-                    v = gte / (1.0f + expf(-gte)) * acc2[i][j][r];
-                }
-                if (EPI == PCB_EPI_SCALE_ADD) {
-                    float* y = (float*)a.y + (int64_t)m * a.ldy + n;
-                    const float b0 = a.base ? a.base[(int64_t)m * a.ldbase + n] : *y;
-                    *y = b0 + cs * v;
-                    continue;
-                }
-                if (a.split_n > 0 && n >= a.split_n) {
-                    const int c = n - a.split_n;
-                    E* y = (E*)a.y2 + a.row_off2[m] + (int64_t)(c / a.head_dim2) * a.head_stride2 + c % a.head_dim2;
-                    *y = from_f32<E>(v);
-                    continue;
-                }
-                const int64_t at = (int64_t)(a.row_dst ? a.row_dst[m] : m) * a.ldy + n;
-                if (a.out_f32)
-                    ((float*)a.y)[at] = v;
-                else
-                    ((E*)a.y)[at] = from_f32<E>(v);
+                if (m < m_hi) emit<E, EPI>(a, m, n, acc[i][j][r], TWO ? acc2[i][j][r] : 0.0f, bv, cs);
             }
+    }
+}
+
+// ---- few rows: the weights stream once, straight from memory into the matrix cores --------------------------------------------
+// Workgroup = 16 result columns x up to 16 rows; its four waves split the contraction (k-step s goes to wave s % 4) and add their
+// partial tiles through LDS.  No LDS staging: a lane's B fragment is 16 contiguous bytes of its weight row, its A fragment 16
+// bytes of its activation row (a handful of rows that stay in cache).
+template <typename E>
+__device__ __forceinline__ void scale_frag(Frag<E>& f, float s);
+template <>
+__device__ __forceinline__ void scale_frag<bf16_t>(Frag<bf16_t>& f, float s) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint32_t w = f.v[e];
+        const uint32_t lo = bf16_bits(s * __uint_as_float(w << 16)), hi = bf16_bits(s * __uint_as_float(w & 0xffff0000u));
+        f.v[e] = lo | (hi << 16);
+    }
+}
+template <>
+__device__ __forceinline__ void scale_frag<float>(Frag<float>& f, float s) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f.v[e] *= s;
+}
+
+template <typename E, int EPI>
+__global__ __launch_bounds__(256) void linear_skinny_kernel(pcb_linear_args a) {
+    constexpr bool TWO = EPI == PCB_EPI_SILU_MUL;
+    constexpr int CE = Tile<E>::CE;
+    __shared__ f4 red[TWO ? 2 : 1][4][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, group = lane >> 4, l15 = lane & 15;
+    const int K = a.K, N = a.N;
+    int g = 0, m_lo, m_hi;
+    if (a.n_groups > 0) {
+        int t = blockIdx.y;
+        m_lo = -1;
+        for (g = 0; g < a.n_groups; ++g) {
+            const int lo = a.group_off[g], hi = a.group_off[g + 1];
+            const int nt = (hi - lo + 15) / 16;
+            if (t < nt) {
+                m_lo = lo + t * 16;
+                m_hi = hi;
+                break;
+            }
+            t -= nt;
+        }
+        if (m_lo < 0) return;
+    } else {
+        m_lo = blockIdx.y * 16;
+        m_hi = a.M;
+        if (m_lo >= m_hi) return;
+    }
+    const int n_lo = blockIdx.x * 16;
+    const E* W = (const E*)a.w + (int64_t)g * a.w_group_stride;
+    const E* W2 = TWO ? (const E*)a.w2 + (int64_t)g * a.w_group_stride : nullptr;
+    const E* X = (const E*)a.x;
+    const bool vec = (K % CE == 0) && (a.ldx % CE == 0) && (a.ldw % CE == 0) && (((uintptr_t)X | (uintptr_t)W | (uintptr_t)W2) % 16 == 0);
+    const int n_b = n_lo + l15, m_a = m_lo + l15;
+    const bool b_ok = n_b < N, a_ok = m_a < m_hi;
+    const E* wrow = W + (int64_t)(b_ok ? n_b : 0) * a.ldw;
+    const E* wrow2 = TWO ? W2 + (int64_t)(b_ok ? n_b : 0) * a.ldw : nullptr;
+    const E* xrow = X + (int64_t)(a_ok ? (a.row_src ? a.row_src[m_a] : m_a) : 0) * a.ldx;
+    const bool scaled = a.row_scale != nullptr;
+    const float xs = (scaled && a_ok) ? a.row_scale[m_a] : 1.0f;
+    f4 acc = f4{0.f, 0.f, 0.f, 0.f}, acc2 = f4{0.f, 0.f, 0.f, 0.f};
+    const int nsteps = (K + 31) / 32;
+#pragma unroll 4
+    for (int st = wave; st < nsteps; st += 4) {
+        const int k0 = 32 * st;
+        Frag<E> fa = load_frag(xrow + k0, group, a_ok ? K - k0 : 0, vec);
+        if (scaled) scale_frag<E>(fa, xs);
+        const Frag<E> fb = load_frag(wrow + k0, group, b_ok ? K - k0 : 0, vec);
+        acc = mma(fa, fb, acc);
+        if (TWO) {
+            const Frag<E> fb2 = load_frag(wrow2 + k0, group, b_ok ? K - k0 : 0, vec);
+            acc2 = mma(fa, fb2, acc2);
+        }
+    }
+    red[0][wave][lane] = acc;
+    if (TWO) red[1][wave][lane] = acc2;
+    __syncthreads();
+    if (wave != 0) return;
+    acc = red[0][0][lane] + red[0][1][lane] + red[0][2][lane] + red[0][3][lane];
+    if (TWO) acc2 = red[1][0][lane] + red[1][1][lane] + red[1][2][lane] + red[1][3][lane];
+    const int n = n_lo + l15;
+    if (n >= N) return;
+    const E* bias = (const E*)a.bias;
+    const float bv = bias ? to_f32(bias[n]) : 0.0f;
+    const float cs = (EPI == PCB_EPI_SCALE_ADD) ? a.col_scale[n] : 0.0f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int m = m_lo + 4 * group + r;
+        if (m < m_hi) emit<E, EPI>(a, m, n, acc[r], acc2[r], bv, cs);
     }
 }
 
@@ -211,6 +305,20 @@ int dispatch(const pcb_linear_args& a, hipStream_t stream) {
     // rows per group decide the row tile: many rows -> 128-row panels, few -> 32-row panels (the weights stream once)
     const int rows = a.n_groups > 0 ? pcb_ceil_div(a.M, a.n_groups) : a.M;
     const bool big = rows > 64;
+    if (rows <= 16) {
+        const dim3 grid(pcb_ceil_div(a.N, 16), pcb_ceil_div(a.M, 16) + (a.n_groups > 0 ? a.n_groups : 0));
+        switch (a.epilogue) {
+            case PCB_EPI_STORE:
+                hipLaunchKernelGGL((linear_skinny_kernel<E, PCB_EPI_STORE>), grid, dim3(256), 0, stream, a);
+                break;
+            case PCB_EPI_SILU_MUL:
+                hipLaunchKernelGGL((linear_skinny_kernel<E, PCB_EPI_SILU_MUL>), grid, dim3(256), 0, stream, a);
+                break;
+            default:
+                hipLaunchKernelGGL((linear_skinny_kernel<E, PCB_EPI_SCALE_ADD>), grid, dim3(256), 0, stream, a);
+        }
+        return pcb_check_launch("linear_skinny_kernel");
+    }
     switch (a.epilogue) {
         case PCB_EPI_STORE:
             return big ? launch<E, PCB_EPI_STORE, 4, 4>(a, stream) : launch<E, PCB_EPI_STORE, 1, 2>(a, stream);
