@@ -149,6 +149,8 @@ typedef struct pcb_attn_talk_args {
     int64_t ldo;
     const int32_t* tiles64; /* optional: the same rows cut into tiles of up to 64 queries (same record) for the value pass */
     int32_t n_tiles64;
+    int32_t max_tile_rows; /* an upper bound of the tiles' query rows when the host knows one (0: unknown); <= 4 selects the
+                              value pass written for decoding */
 } pcb_attn_talk_args;
 int32_t pcb_attn_talk_band(int32_t window, int32_t max_kv_len);
 int pcb_attn_talk(const pcb_attn_talk_args* a, void* stream);

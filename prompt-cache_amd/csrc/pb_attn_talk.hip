@@ -238,6 +238,109 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
     }
 }
 
+// ---- 2b. values for tiles of at most 4 rows (decoding) -------------------------------------------------------------------------
+// A row's output is a weighted sum of key rows: no matrix core needed, and nothing to transpose.  Thread = (column d, key slice);
+// it walks its slice's keys with coalesced loads (a key row is contiguous over d), multiplies by the rows' weights from LDS
+// (fp32, not rounded) and the slices meet in LDS at the end.
+constexpr int FEW_ROWS = 4, FEW_KEYS = 512;
+
+template <typename E>
+__global__ __launch_bounds__(256) void talk_values_few_kernel(pcb_attn_talk_args a, int band, const int32_t* tiles) {
+    __shared__ float row_m[FEW_ROWS], row_inv[FEW_ROWS];
+    __shared__ float P[FEW_ROWS][FEW_KEYS];
+    __shared__ float red[FEW_ROWS][256];
+    const int H = a.H, D = a.head_dim, rep = H / a.Hkv;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const TileRec t = reinterpret_cast<const TileRec*>(tiles)[blockIdx.x];
+    const int h = blockIdx.y;
+    const int window = a.window > 0 ? a.window : 0x3fffffff;
+    const int i_last = t.q0 + t.nq - 1;
+    const int j_min = t.q0 - window + 1 > 0 ? t.q0 - window + 1 : 0;
+    const float* __restrict__ S = a.scratch + ((int64_t)t.row0 * H + h) * band;
+    const int64_t s_row = (int64_t)H * band;
+    for (int r = wave; r < t.nq; r += 4) {
+        const int i = t.q0 + r;
+        const int n = i + 1 < window ? i + 1 : window;
+        const float* sr = S + r * s_row;
+        float m = a.sink ? 0.0f : -INFINITY;
+        for (int d = lane; d < n; d += 64) m = fmaxf(m, sr[d]);
+        m = wave_max(m);
+        float l = 0.0f;
+        for (int d = lane; d < n; d += 64) l += expf(sr[d] - m);
+        l = wave_sum(l);
+        if (a.sink) l += expf(-m);
+        if (lane == 0) row_m[r] = m, row_inv[r] = 1.0f / l;
+    }
+    __syncthreads();
+    const E* __restrict__ V = (const E*)a.cache + (int64_t)t.slot * a.slot_stride + (int64_t)(h / rep) * a.head_stride;
+    // wide form: a thread owns one 16-byte chunk of the key rows (CE columns) and every (256 / chunks)-th key
+    constexpr int CE = 16 / sizeof(E);
+    const bool wide = D % CE == 0 && D / CE <= 256 && a.head_stride % CE == 0 && a.slot_stride % CE == 0 && ((uintptr_t)a.cache % 16 == 0);
+    const int cols = wide ? D / CE : D;               // thread columns; D <= 256
+    const int n_slices = 256 / cols;
+    const int dcol = tid % cols, slice = tid / cols;
+    const bool active = slice < n_slices;
+    float acc[FEW_ROWS][CE];
+#pragma unroll
+    for (int r = 0; r < FEW_ROWS; ++r)
+#pragma unroll
+        for (int i = 0; i < CE; ++i) acc[r][i] = 0.0f;
+    for (int j0 = j_min; j0 <= i_last; j0 += FEW_KEYS) {
+        const int n = i_last - j0 + 1 < FEW_KEYS ? i_last - j0 + 1 : FEW_KEYS;
+        for (int e = tid; e < FEW_ROWS * FEW_KEYS; e += 256) {
+            const int r = e / FEW_KEYS, kk = e % FEW_KEYS;
+            const int dist = t.q0 + r - (j0 + kk);
+            float p = 0.0f;
+            if (r < t.nq && kk < n && dist >= 0 && dist < window) p = expf(S[r * s_row + dist] - row_m[r]) * row_inv[r];
+            P[r][kk] = p;
+        }
+        __syncthreads();
+        if (active && wide) {
+#pragma unroll 4
+            for (int kk = slice; kk < n; kk += n_slices) {
+                __attribute__((aligned(16))) E tmp[CE];
+                *reinterpret_cast<u32x4*>(tmp) = *reinterpret_cast<const u32x4*>(V + (int64_t)(j0 + kk) * D + dcol * CE);
+#pragma unroll
+                for (int r = 0; r < FEW_ROWS; ++r) {
+                    const float p = P[r][kk];
+#pragma unroll
+                    for (int i = 0; i < CE; ++i) acc[r][i] += p * to_f32(tmp[i]);
+                }
+            }
+        } else if (active) {
+#pragma unroll 4
+            for (int kk = slice; kk < n; kk += n_slices) {
+                const float v = to_f32(V[(int64_t)(j0 + kk) * D + dcol]);
+#pragma unroll
+                for (int r = 0; r < FEW_ROWS; ++r) acc[r][0] += P[r][kk] * v;
+            }
+        }
+        __syncthreads();
+    }
+    // the slices meet in LDS, one column chunk element at a time (red is [rows][256])
+    E* O = (E*)a.out;
+    const int per = wide ? CE : 1;
+    for (int i = 0; i < per; ++i) {
+#pragma unroll
+        for (int r = 0; r < FEW_ROWS; ++r) {
+            float v = 0.0f;
+#pragma unroll
+            for (int i2 = 0; i2 < CE; ++i2)
+                if (i2 == i) v = acc[r][i2];
+            red[r][tid] = active ? v : 0.0f;
+        }
+        __syncthreads();
+        if (tid < cols) {
+            for (int r = 0; r < t.nq; ++r) {
+                float v = 0.0f;
+                for (int sl = 0; sl < n_slices; ++sl) v += red[r][sl * cols + tid];
+                O[(int64_t)(t.row0 + r) * a.ldo + h * D + tid * per + i] = from_f32<E>(v);
+            }
+        }
+        __syncthreads();
+    }
+}
+
 template <typename E, int HMAX>
 void launch_scores(const pcb_attn_talk_args& a, int band, hipStream_t stream) {
     // the tile's queries wait in LDS when 16 rows of all heads fit beside the kernel's own tables (160 KiB per workgroup)
@@ -273,6 +376,10 @@ int run(const pcb_attn_talk_args& a, int band, hipStream_t stream) {
     const size_t lds = (size_t)D16 * (32 + 16 / sizeof(E)) * sizeof(E);
     const int32_t* tiles = a.tiles64 ? a.tiles64 : a.tiles;
     const dim3 grid(a.tiles64 ? a.n_tiles64 : a.n_tiles, H);
+    if (a.max_tile_rows > 0 && a.max_tile_rows <= FEW_ROWS) {
+        hipLaunchKernelGGL((talk_values_few_kernel<E>), grid, dim3(256), 0, stream, a, band, tiles);
+        return pcb_check_launch("talk_values_few_kernel");
+    }
     if (D16 <= 64)
         hipLaunchKernelGGL((talk_values_kernel<E, 4>), grid, dim3(256), lds, stream, a, band, tiles);
     else if (D16 <= 128)

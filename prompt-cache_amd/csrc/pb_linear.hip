@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256) void linear_kernel(pcb_linear_args a) {
 }
 
 // ---- few rows: the weights stream once, straight from memory into the matrix cores --------------------------------------------
-// Workgroup = 16 result columns x up to 16 rows; its four waves split the contraction (k-step s goes to wave s % 4) and add their
+// Workgroup = 16 result columns x up to 16 rows; its eight waves split the contraction (k-step s goes to wave s % 8) and add their
 // partial tiles through LDS.  No LDS staging: a lane's B fragment is 16 contiguous bytes of its weight row, its A fragment 16
 // bytes of its activation row (a handful of rows that stay in cache).
 template <typename E>
@@ -221,11 +221,13 @@ __device__ __forceinline__ void scale_frag<float>(Frag<float>& f, float s) {
     for (int e = 0; e < 8; ++e) f.v[e] *= s;
 }
 
+constexpr int SKW = 8;          // waves of a few-row workgroup
+
 template <typename E, int EPI>
-__global__ __launch_bounds__(256) void linear_skinny_kernel(pcb_linear_args a) {
+__global__ __launch_bounds__(64 * SKW) void linear_skinny_kernel(pcb_linear_args a) {
     constexpr bool TWO = EPI == PCB_EPI_SILU_MUL;
     constexpr int CE = Tile<E>::CE;
-    __shared__ f4 red[TWO ? 2 : 1][4][64];
+    __shared__ f4 red[TWO ? 2 : 1][SKW][64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, group = lane >> 4, l15 = lane & 15;
     const int K = a.K, N = a.N;
     int g = 0, m_lo, m_hi;
@@ -262,8 +264,8 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(pcb_linear_args a) {
     const float xs = (scaled && a_ok) ? a.row_scale[m_a] : 1.0f;
     f4 acc = f4{0.f, 0.f, 0.f, 0.f}, acc2 = f4{0.f, 0.f, 0.f, 0.f};
     const int nsteps = (K + 31) / 32;
-#pragma unroll 4
-    for (int st = wave; st < nsteps; st += 4) {
+#pragma unroll 8
+    for (int st = wave; st < nsteps; st += SKW) {
         const int k0 = 32 * st;
         Frag<E> fa = load_frag(xrow + k0, group, a_ok ? K - k0 : 0, vec);
         if (scaled) scale_frag<E>(fa, xs);
@@ -278,8 +280,13 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(pcb_linear_args a) {
     if (TWO) red[1][wave][lane] = acc2;
     __syncthreads();
     if (wave != 0) return;
-    acc = red[0][0][lane] + red[0][1][lane] + red[0][2][lane] + red[0][3][lane];
-    if (TWO) acc2 = red[1][0][lane] + red[1][1][lane] + red[1][2][lane] + red[1][3][lane];
+    acc = red[0][0][lane];
+    if (TWO) acc2 = red[1][0][lane];
+#pragma unroll
+    for (int w = 1; w < SKW; ++w) {
+        acc += red[0][w][lane];
+        if (TWO) acc2 += red[1][w][lane];
+    }
     const int n = n_lo + l15;
     if (n >= N) return;
     const E* bias = (const E*)a.bias;
@@ -309,13 +316,13 @@ int dispatch(const pcb_linear_args& a, hipStream_t stream) {
         const dim3 grid(pcb_ceil_div(a.N, 16), pcb_ceil_div(a.M, 16) + (a.n_groups > 0 ? a.n_groups : 0));
         switch (a.epilogue) {
             case PCB_EPI_STORE:
-                hipLaunchKernelGGL((linear_skinny_kernel<E, PCB_EPI_STORE>), grid, dim3(256), 0, stream, a);
+                hipLaunchKernelGGL((linear_skinny_kernel<E, PCB_EPI_STORE>), grid, dim3(64 * SKW), 0, stream, a);
                 break;
             case PCB_EPI_SILU_MUL:
-                hipLaunchKernelGGL((linear_skinny_kernel<E, PCB_EPI_SILU_MUL>), grid, dim3(256), 0, stream, a);
+                hipLaunchKernelGGL((linear_skinny_kernel<E, PCB_EPI_SILU_MUL>), grid, dim3(64 * SKW), 0, stream, a);
                 break;
             default:
-                hipLaunchKernelGGL((linear_skinny_kernel<E, PCB_EPI_SCALE_ADD>), grid, dim3(256), 0, stream, a);
+                hipLaunchKernelGGL((linear_skinny_kernel<E, PCB_EPI_SCALE_ADD>), grid, dim3(64 * SKW), 0, stream, a);
         }
         return pcb_check_launch("linear_skinny_kernel");
     }

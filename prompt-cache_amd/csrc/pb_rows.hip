@@ -20,10 +20,10 @@ PCB_EXPORT const char* pcb_last_error_string(void) { return g_err; }
 namespace {
 using namespace pcb;
 
-// block-wide sum of NV values per thread (256 threads); every thread gets the totals
+// block-wide sum of NV values per thread; every thread gets the totals.  red: [waves * NV]
 template <int NV>
-__device__ __forceinline__ void block_sum(float (&v)[NV], float* red /* [4 * NV] */) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+__device__ __forceinline__ void block_sum(float (&v)[NV], float* red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
 #pragma unroll
     for (int i = 0; i < NV; ++i) v[i] = wave_sum(v[i]);
     __syncthreads();
@@ -33,7 +33,11 @@ __device__ __forceinline__ void block_sum(float (&v)[NV], float* red /* [4 * NV]
     }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < NV; ++i) v[i] = red[i] + red[NV + i] + red[2 * NV + i] + red[3 * NV + i];
+    for (int i = 0; i < NV; ++i) {
+        float t = 0.0f;
+        for (int w = 0; w < waves; ++w) t += red[w * NV + i];
+        v[i] = t;
+    }
 }
 
 template <typename E>
@@ -48,30 +52,30 @@ __global__ __launch_bounds__(256) void embed_rows_kernel(const E* __restrict__ t
 
 // one workgroup per output row; the row is held in LDS between the sum and the norms (width * 4 bytes of dynamic LDS)
 template <typename E>
-__global__ __launch_bounds__(256) void mix_norm_kernel(pcb_mix_norm_args a) {
+__global__ __launch_bounds__(1024) void mix_norm_kernel(pcb_mix_norm_args a) {
     extern __shared__ float row[];
-    __shared__ float red[8];
+    __shared__ float red[16];
     const int r = blockIdx.x;
     const int64_t src = a.rows ? a.rows[r] : r;
     const int W = a.width;
     float ss[1] = {0.0f};
-    for (int c = threadIdx.x; c < W; c += 256) {
-        float x;
-        if (a.n_terms > 0) {
-            x = 0.0f;
-            for (int j = 0; j < a.n_terms; ++j) x += a.coef[j] * a.hist[j * a.hist_stride + src * W + c];
-        } else {
-            x = a.hist[src * W + c];
-        }
+    // (streams and coefficients are read through restrict-qualified pointers: the stores to x_out must not fence the loads)
+    const float* __restrict__ hist = a.hist + src * W;
+    const float* __restrict__ coef = a.coef;
+    float* __restrict__ xo = a.x_out ? a.x_out + (int64_t)r * W : nullptr;
+    const int nt = a.n_terms;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        float x = nt > 0 ? 0.0f : hist[c];
+        for (int j = 0; j < nt; ++j) x += coef[j] * hist[j * a.hist_stride + c];
         row[c] = x;
-        if (a.x_out) a.x_out[(int64_t)r * W + c] = x;
+        if (xo) xo[c] = x;
         ss[0] += x * x;
     }
     block_sum<1>(ss, red);
     const float inv = 1.0f / sqrtf(ss[0] / (float)W + a.eps);
     E* o1 = (E*)a.out1;
     E* o2 = (E*)a.out2;
-    for (int c = threadIdx.x; c < W; c += 256) {
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
         const float x = row[c] * inv;
         if (o1) o1[(int64_t)r * W + c] = from_f32<E>(x * a.gain1[c]);
         if (o2) o2[(int64_t)r * W + c] = from_f32<E>(x * a.gain2[c]);
@@ -79,13 +83,13 @@ __global__ __launch_bounds__(256) void mix_norm_kernel(pcb_mix_norm_args a) {
 }
 
 template <typename E>
-__global__ __launch_bounds__(256) void polynorm_kernel(const float* __restrict__ z, const float* __restrict__ coef, E* __restrict__ out,
+__global__ __launch_bounds__(1024) void polynorm_kernel(const float* __restrict__ z, const float* __restrict__ coef, E* __restrict__ out,
                                                        float eps, int ff) {
-    __shared__ float red[12];
+    __shared__ float red[48];
     const int64_t r = blockIdx.x;
     const float* zr = z + r * ff;
     float s[3] = {0.0f, 0.0f, 0.0f};
-    for (int c = threadIdx.x; c < ff; c += 256) {
+    for (int c = threadIdx.x; c < ff; c += blockDim.x) {
         const float v = zr[c], v2 = v * v, v3 = v2 * v;
         s[0] += v2;
         s[1] += v2 * v2;
@@ -96,7 +100,7 @@ __global__ __launch_bounds__(256) void polynorm_kernel(const float* __restrict__
     const float i2 = coef[1] / sqrtf(s[1] / (float)ff + eps);
     const float i3 = coef[2] / sqrtf(s[2] / (float)ff + eps);
     const float c3 = coef[3];
-    for (int c = threadIdx.x; c < ff; c += 256) {
+    for (int c = threadIdx.x; c < ff; c += blockDim.x) {
         const float v = zr[c], v2 = v * v;
         out[r * ff + c] = from_f32<E>(i1 * v + i2 * v2 + i3 * (v2 * v) + c3);
     }
@@ -203,10 +207,12 @@ PCB_EXPORT int pcb_mix_norm(const pcb_mix_norm_args* a, void* stream) {
     PCB_REQUIRE(a->hist && (a->n_terms == 0 || a->coef) && (!a->out1 || a->gain1) && (!a->out2 || a->gain2), PCB_ERR_ARG,
                 "pcb_mix_norm: null pointer");
     const size_t lds = (size_t)a->width * sizeof(float);
+    // few rows: a row's columns are spread over up to 1024 threads (the loads of a thread's columns are a dependent chain)
+    const dim3 threads(a->n_rows <= 512 && a->width > 1024 ? 1024 : 256);
     if (a->dtype == PCB_BF16)
-        hipLaunchKernelGGL(mix_norm_kernel<bf16_t>, dim3(a->n_rows), dim3(256), lds, (hipStream_t)stream, *a);
+        hipLaunchKernelGGL(mix_norm_kernel<bf16_t>, dim3(a->n_rows), threads, lds, (hipStream_t)stream, *a);
     else
-        hipLaunchKernelGGL(mix_norm_kernel<float>, dim3(a->n_rows), dim3(256), lds, (hipStream_t)stream, *a);
+        hipLaunchKernelGGL(mix_norm_kernel<float>, dim3(a->n_rows), threads, lds, (hipStream_t)stream, *a);
     return pcb_check_launch("mix_norm_kernel");
 }
 
@@ -215,10 +221,11 @@ PCB_EXPORT int pcb_polynorm(const float* z, const float* coef, void* out, int32_
     PCB_REQUIRE(PCB_DTYPE_OK(dtype) && n_rows >= 0 && ff > 0, PCB_ERR_ARG, "pcb_polynorm: bad sizes");
     if (n_rows == 0) return PCB_OK;
     PCB_REQUIRE(z && coef && out, PCB_ERR_ARG, "pcb_polynorm: null pointer");
+    const dim3 threads(n_rows <= 512 && ff > 1024 ? 1024 : 256);
     if (dtype == PCB_BF16)
-        hipLaunchKernelGGL(polynorm_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, z, coef, (bf16_t*)out, eps, ff);
+        hipLaunchKernelGGL(polynorm_kernel<bf16_t>, dim3(n_rows), threads, 0, (hipStream_t)stream, z, coef, (bf16_t*)out, eps, ff);
     else
-        hipLaunchKernelGGL(polynorm_kernel<float>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, z, coef, (float*)out, eps, ff);
+        hipLaunchKernelGGL(polynorm_kernel<float>, dim3(n_rows), threads, 0, (hipStream_t)stream, z, coef, (float*)out, eps, ff);
     return pcb_check_launch("polynorm_kernel");
 }
 

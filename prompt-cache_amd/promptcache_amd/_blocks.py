@@ -47,7 +47,7 @@ class AttnTalkArgs(C.Structure):
                 ("H", _i32), ("Hkv", _i32), ("head_dim", _i32), ("scale", _f32), ("window", _i32), ("max_kv_len", _i32),
                 ("slopes", _vp), ("talk", _vp), ("sink", _i32),
                 ("scratch", _vp), ("scratch_floats", _i64), ("out", _vp), ("ldo", _i64),
-                ("tiles64", _vp), ("n_tiles64", _i32)]
+                ("tiles64", _vp), ("n_tiles64", _i32), ("max_tile_rows", _i32)]
 
 
 # name -> (restype, argtypes); mirrors include/promptcache_blocks.h one to one
@@ -234,7 +234,8 @@ def attn_talk_band(window: int, max_kv_len: int) -> int:
 
 def attn_talk(q: torch.Tensor, tiles: torch.Tensor, n_tiles: int, cache: torch.Tensor, slot_stride: int, head_stride: int,
               H: int, Hkv: int, head_dim: int, scale: float, window: int, max_kv_len: int, slopes, talk, sink: bool,
-              scratch: torch.Tensor, out: torch.Tensor, tiles64: Optional[torch.Tensor] = None, n_tiles64: int = 0) -> None:
+              scratch: torch.Tensor, out: torch.Tensor, tiles64: Optional[torch.Tensor] = None, n_tiles64: int = 0,
+              max_tile_rows: int = 0) -> None:
     _want(tiles, torch.int32, "attn_talk tiles"); _want(scratch, torch.float32, "attn_talk scratch")
     assert q.dtype == cache.dtype == out.dtype and q.is_contiguous() and out.is_contiguous() and cache.is_cuda
     assert tiles.numel() >= 4 * n_tiles and q.shape[-1] == H * head_dim and out.shape[-1] == H * head_dim
@@ -245,7 +246,8 @@ def attn_talk(q: torch.Tensor, tiles: torch.Tensor, n_tiles: int, cache: torch.T
         _want(talk, torch.float32, "attn_talk talk"); assert talk.numel() == H * H
     a = AttnTalkArgs(C.sizeof(AttnTalkArgs), _code(q), _p(q), q.shape[-1], _p(tiles), n_tiles, _p(cache), slot_stride,
                      head_stride, H, Hkv, head_dim, float(scale), int(window), int(max_kv_len), _p(slopes), _p(talk), int(sink),
-                     _p(scratch), scratch.numel(), _p(out), out.shape[-1], _p(tiles64), n_tiles64 if tiles64 is not None else 0)
+                     _p(scratch), scratch.numel(), _p(out), out.shape[-1], _p(tiles64), n_tiles64 if tiles64 is not None else 0,
+                     int(max_tile_rows))
     if tiles64 is not None:
         _want(tiles64, torch.int32, "attn_talk tiles64")
         assert tiles64.numel() >= 4 * n_tiles64 > 0

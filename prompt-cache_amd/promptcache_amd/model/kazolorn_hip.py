@@ -22,6 +22,7 @@ and the logits are ``head . rms(sum_j dwa_last[j] X_j) g`` for the rows that wer
 """
 from __future__ import annotations
 
+import os
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -103,6 +104,9 @@ class KazolornHIP:
             self.layers.append(ent)
         self._buf = {}
         self.default_arena: Optional[SlotArena] = None
+        self.use_graphs = os.environ.get("PC_KZ_GRAPHS", "1") != "0"      # one-token steps replay a captured hipGraph
+        self._graphs = {}
+        self.max_graphs = 16
 
     # ---- cache -------------------------------------------------------------------------------------------------------------
     def new_arena(self, slots: int, cap: int) -> SlotArena:
@@ -161,10 +165,17 @@ class KazolornHIP:
         tiles = np.asarray(tiles, dtype=np.int32).reshape(-1, 4)
         tiles64 = np.asarray([(s, st + q, min(64, c - q), int(row0[b]) + q) for b, (s, st, c) in enumerate(zip(slots, starts, counts))
                               for q in range(0, c, 64)], dtype=np.int32).reshape(-1, 4)
-        want_rows = np.asarray([int(row0[b]) + int(w) for b, ws in enumerate(want) for w in ws], dtype=np.int32)
         for b, ws in enumerate(want):
             if any(not 0 <= int(w) < counts[b] for w in ws):
                 raise ValueError("a wanted place lies outside its request's tokens")
+        # one-token steps run as a captured graph whose launches have fixed sizes: logits of every row, picked from afterwards
+        graphed = (self.use_graphs and T <= self.GRAPH_MAX_ROWS and all(c == 1 for c in counts) and num_layers is None
+                   and not return_streams)
+        picked = None
+        if graphed and any(len(ws) != 1 for ws in want):
+            picked = [b for b, ws in enumerate(want) for _ in ws]
+        want_rows = np.arange(T, dtype=np.int32) if graphed else \
+            np.asarray([int(row0[b]) + int(w) for b, ws in enumerate(want) for w in ws], dtype=np.int32)
         sigs = sorted({(l.kv_heads, l.dim) for l in self.config.layers})
         offs = np.stack([row_slot * (g * arena.cap * d) + row_pos * d for g, d in sigs]) if T else np.zeros((len(sigs), 0), np.int64)
         n32 = T + tiles.size + want_rows.size + tiles64.size
@@ -172,12 +183,30 @@ class KazolornHIP:
         o64 = (n32 * 4 + 7) // 8 * 8
         blob[:n32 * 4].view(np.int32)[:] = np.concatenate([ids, tiles.reshape(-1), want_rows, tiles64.reshape(-1)])
         blob[o64:o64 + offs.size * 8].view(np.int64)[:] = offs.reshape(-1)
-        dblob = torch.from_numpy(blob).to(dev)
-        d32 = dblob[:n32 * 4].view(torch.int32)
-        ids_d, tiles_d, want_d = d32[:T], d32[T:T + tiles.size], d32[T + tiles.size:T + tiles.size + want_rows.size]
-        tiles64_d = d32[T + tiles.size + want_rows.size:]
-        offs_d = dblob[o64:o64 + offs.size * 8].view(torch.int64).view(len(sigs), T)
+        n_want = int(want_rows.size)
+        res = self._decode_graphed(arena, T, blob, n32, o64, sigs) if graphed else None
+        if res is None:
+            dblob = torch.from_numpy(blob).to(dev)
+            logits = torch.empty((n_want, V), dtype=f32, device=dev)
+            res = self._run(arena, T, dblob, n32, o64, sigs, tiles, tiles.shape[0], tiles64.shape[0], n_want, max_kv, logits,
+                            num_layers, return_streams)
+        for s_, c in zip(slots, counts):
+            arena.lengths[s_] += c
+        if picked is not None:
+            res = res[torch.as_tensor(picked, dtype=torch.long, device=dev)] if picked else res[:0]
+        return res
 
+    def _run(self, arena, T, dblob, n32, o64, sigs, tiles, n_tiles, n64, n_want, max_kv, logits, num_layers=None,
+             return_streams=False):
+        """The device side of a step: every launch of the forward, reading the step's tables from ``dblob`` (token ids, the two
+        tile tables, wanted rows as int32, then the cache offsets of every row as int64)."""
+        dev, E, f32 = self.device, self.dtype, torch.float32
+        W, V = self.W, self.V
+        d32 = dblob[:n32 * 4].view(torch.int32)
+        ids_d, tiles_d = d32[:T], d32[T:T + 4 * n_tiles]
+        want_d = d32[T + 4 * n_tiles:T + 4 * n_tiles + n_want]
+        tiles64_d = d32[T + 4 * n_tiles + n_want:T + 4 * n_tiles + n_want + 4 * n64]
+        offs_d = dblob[o64:o64 + len(sigs) * T * 8].view(torch.int64).view(len(sigs), T)
         layers = self.layers if num_layers is None else self.layers[:num_layers]
         L = len(layers)
         hist = self._scratch("hist", (L + 1) * T * W, f32)[:(L + 1) * T * W].view(L + 1, T, W)
@@ -205,7 +234,8 @@ class KazolornHIP:
             B.linear(h1, lw["wqk"], q, M=T, bias=lw["bqk"], split_n=HD, y2=plane, row_off2=offs_d[sigs.index((l.kv_heads, l.dim))],
                      head_dim2=l.dim, head_stride2=arena.head_stride(i))
             att = self._mat("att", T, HD, E)
-            self._attention(q, att, tiles, tiles_d, tiles64_d, tiles64.shape[0], plane, arena, i, l, lw, max_kv)
+            self._attention(q, att, tiles, n_tiles, tiles_d, tiles64_d, n64, plane, arena, i, l, lw, max_kv,
+                            max_rows=1 if n_tiles == T else (int(tiles[:, 2].max()) if tiles is not None and n64 == n_tiles else 0))
             B.linear(att, lw["wo"], hist[i + 1], M=T, epilogue=B.EPI_SCALE_ADD, bias=lw["bo"], base=base, col_scale=lw["ls1"])
             if l.mlp_kind == "dense":
                 z = self._mat("z", T, l.ff, f32)
@@ -230,8 +260,6 @@ class KazolornHIP:
                 B.linear(gact, lw["down"], pair, M=P, row_dst=row_dst, group_off=goff, n_groups=l.experts)
                 B.moe_combine(pair, lw["ls2"], hist[i + 1], T, l.top)
 
-        n_want = int(want_rows.size)
-        logits = torch.empty((n_want, V), dtype=f32, device=dev)
         if streams is not None:
             B.mix_norm(hist, L + 1, layers[-1]["dwa"], None, None, x_out=x, eps=eps, n_rows=T)
             streams[L - 1].copy_(x)
@@ -239,19 +267,63 @@ class KazolornHIP:
             hn = self._mat("hn", n_want, W, E)
             B.mix_norm(hist, L + 1, layers[-1]["dwa"], self.final_norm, hn, rows=want_d, eps=eps, n_rows=n_want)
             B.linear(hn, self.head, logits, M=n_want)
-        for s, c in zip(slots, counts):
-            arena.lengths[s] += c
         return (logits, streams) if return_streams else logits
 
-    def _attention(self, q, att, tiles, tiles_d, tiles64_d, n64, plane, arena, i, l, lw, max_kv):
+    # ---- decode steps as captured graphs -----------------------------------------------------------------------------------------
+    GRAPH_MAX_ROWS = 64
+
+    def _decode_graphed(self, arena, T, blob, n32, o64, sigs):
+        """A step of T requests with one token each, replayed from a hipGraph captured per (T, arena planes).  What changes between
+        steps -- tokens, slots, positions -- lives in the step's tables, which the graph reads from a device block that one copy
+        from pinned memory refreshes; every launch dimension is sized for the arena's row capacity instead of the current
+        lengths.  Returns None when the score band of such a launch would be too large (the caller then runs eagerly)."""
+        cap = arena.cap
+        worst = max(16 * T * l.heads * B.attn_talk_band(l.window, cap) for l in self.config.layers)
+        if worst > ATTN_SCRATCH_FLOATS // 4:
+            return None
+        key = (T, id(arena), arena.generation)
+        ent = self._graphs.pop(key, None)
+        if ent is None:
+            for k in [k for k in self._graphs if k[1] == id(arena) and k[2] != arena.generation]:
+                del self._graphs[k]                               # graphs over planes that have moved
+            while len(self._graphs) >= self.max_graphs:
+                self._graphs.pop(next(iter(self._graphs)))
+            ent = dict(graph=None, bufs={}, host=torch.empty(blob.size, dtype=torch.uint8, pin_memory=True),
+                       dev=torch.empty(blob.size, dtype=torch.uint8, device=self.device),
+                       logits=torch.empty((T, self.V), dtype=torch.float32, device=self.device), copied=torch.cuda.Event())
+        self._graphs[key] = ent                                   # (re-inserted at the young end)
+        ent["copied"].synchronize()                               # the previous step's upload has left the pinned block
+        ent["host"].numpy()[:] = blob
+        ent["dev"].copy_(ent["host"], non_blocking=True)
+        ent["copied"].record()
+        if ent["graph"] is None:
+            from .llama_hip import prime_graph_capture
+            saved, self._buf = self._buf, ent["bufs"]             # the graph owns its scratch: later, larger steps may regrow the shared one
+            try:
+                args = (arena, T, ent["dev"], n32, o64, sigs, None, T, T, T, cap, ent["logits"])
+                self._run(*args)                                  # eager first: sizes every scratch buffer, and is this step's result
+                torch.cuda.synchronize()
+                prime_graph_capture(self.device)
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    self._run(*args)
+                ent["graph"] = g
+            finally:
+                self._buf = saved
+            # (the eager run already appended this step's keys and produced its logits; the capture itself launches nothing)
+            return ent["logits"].clone()
+        ent["graph"].replay()
+        return ent["logits"].clone()
+
+    def _attention(self, q, att, tiles, n_tiles, tiles_d, tiles64_d, n64, plane, arena, i, l, lw, max_kv, max_rows=0):
         band = B.attn_talk_band(l.window, max_kv)
         per_tile = 16 * l.heads * band
-        n_tiles = tiles.shape[0]
         chunk = max(1, ATTN_SCRATCH_FLOATS // per_tile)
         if n_tiles <= chunk:
             scratch = self._scratch("band", n_tiles * per_tile, torch.float32)
             B.attn_talk(q, tiles_d, n_tiles, plane, arena.slot_stride(i), arena.head_stride(i), l.heads, l.kv_heads, l.dim, l.scale,
-                        l.window, max_kv, lw["slopes"], lw["talk"], True, scratch, att, tiles64=tiles64_d, n_tiles64=n64)
+                        l.window, max_kv, lw["slopes"], lw["talk"], True, scratch, att, tiles64=tiles64_d, n_tiles64=n64,
+                        max_tile_rows=max_rows)
             return
         # too many rows for one score band: several calls, each over a run of tiles with rows counted from the run's first
         scratch = self._scratch("band", chunk * per_tile, torch.float32)
