@@ -6,6 +6,8 @@ cache and once with ``no_cache=True``, printing the two timed intervals of each 
     python demo.py                                   # llama2-7b shape, random weights, synthetic game-like schema
     python demo.py --model falcon --schema my.xml --prompt-file my_prompt.xml
     python demo.py --model /path/to/hf/checkpoint    # real weights + tokenizer when a directory is available
+    python demo.py --model kazolorn                  # the Kazolorn design (random weights), or a directory that holds one:
+                                                     # plain generation, single and batched (no prompt modules for this design)
 
 There is no network on the build / bench machines, so without a checkpoint directory the adapters use seeded random
 weights at the named shape and the deterministic stand-in tokenizer: the text is noise, the timings are real.
@@ -18,15 +20,36 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "prompt-cache_amd"))
 
 from promptcache_amd import CacheEngine, GenerationEngine, GenerationParameters, Prompt, read_file, synth  # noqa: E402
-from promptcache_amd.model import CodeLlama, Falcon, Llama2, Mpt  # noqa: E402
+from promptcache_amd.model import CodeLlama, Falcon, Kazolorn, Llama2, Mpt, load_language_model  # noqa: E402
+from promptcache_amd.model.config import KazolornShape  # noqa: E402
 
 ADAPTERS = {"llama": (Llama2, "llama2-7b"), "codellama": (CodeLlama, "codellama-7b"), "falcon": (Falcon, "falcon-7b"),
             "mpt": (Mpt, "mpt-7b")}
 
 
+def kazolorn_demo(lm, a):
+    """Generation without prompt modules: one request through GenerationEngine, then a few through the batch scheduler."""
+    import time
+    from promptcache_amd import BatchEngine
+    text = open(a.prompt_file).read() if a.prompt_file else "The quick brown fox jumps over the lazy dog. " * 8
+    ids = lm.encode(text) or [1]
+    params = GenerationParameters(temperature=0.0, max_new_tokens=a.max_new_tokens, stop_token_ids=[])
+    last = None
+    for last in GenerationEngine(lm).generate(ids, list(range(len(ids))), params):
+        pass
+    print(f"single : {len(ids):5d} prompt tokens | first forward {last.elapsed_time:8.3f} ms | "
+          f"{a.max_new_tokens} tokens in {last.response_time:8.2f} ms")
+    prompts = [ids, ids[: max(1, len(ids) // 3)], ids[: max(1, len(ids) // 2)] + ids[:5]]
+    t0 = time.perf_counter()
+    out = BatchEngine(lm, max_tokens=a.max_ctx).generate(prompts, params)
+    dt = time.perf_counter() - t0
+    print(f"batched: {len(prompts)} requests of {[len(p) for p in prompts]} tokens | {sum(len(o) for o in out)} tokens in {dt * 1e3:8.2f} ms")
+    print("Assistant:", lm.decode(out[0])[:120])
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--model", default="llama", help="llama | codellama | falcon | mpt | <HF checkpoint directory>")
+    ap.add_argument("--model", default="llama", help="llama | codellama | falcon | mpt | kazolorn | <checkpoint directory>")
     ap.add_argument("--schema", help="PML schema file (default: a synthetic game-like schema, 7 modules)")
     ap.add_argument("--prompt-file", help="PML prompt file referencing the schema")
     ap.add_argument("--max-ctx", type=int, default=5000)
@@ -35,12 +58,16 @@ def main():
     a = ap.parse_args()
 
     if os.path.isdir(a.model):
-        import json
-        arch = json.load(open(os.path.join(a.model, "config.json"))).get("model_type", "llama")
-        lm = {"falcon": Falcon, "mpt": Mpt}.get(arch, Llama2)(a.model)
+        lm = load_language_model(a.model)              # the adapter class follows the directory's config.json
+    elif a.model == "kazolorn":
+        lm = Kazolorn(shape=KazolornShape.uniform(32000, 1024, 4, 8, 2, 128, 256, 4096, experts=8, top=2, expert_ff=1024),
+                      random_init=True)
     else:
         cls, shape = ADAPTERS[a.model]
         lm = cls(shape, random_init=True)
+    if isinstance(lm, Kazolorn):
+        kazolorn_demo(lm, a)
+        return
     preproc = [lm.get_formatter()]
     cache_engine = CacheEngine(a.max_ctx, lm)
     gen_engine = GenerationEngine(lm)

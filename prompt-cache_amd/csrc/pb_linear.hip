@@ -3,8 +3,8 @@
 // layer-scaled accumulation into an fp32 residual stream.
 //
 // Tiling: workgroup = 4 waves in a 2 x 2 grid, a wave owns TM x TN result tiles of 16 x 16, so the workgroup covers
-// (32 TM) x (32 TN) of Y.  Per 32-element k-step the A and B panels go global -> registers -> LDS (the next step's loads are in
-// flight while this step's MFMAs run); waves read their operand fragments from LDS with one 16-byte read per fragment (bf16).
+// (32 TM) x (32 TN) of Y.  Per stage of two 32-element k-steps the A and B panels go global -> registers -> LDS (the next stage's
+// loads are in flight while this stage's MFMAs run); waves read their operand fragments from LDS with one 16-byte read per fragment (bf16).
 #include "pb_common.h"
 
 namespace {
@@ -12,9 +12,10 @@ using namespace pcb;
 
 template <typename E>
 struct Tile {
+    static constexpr int KS = sizeof(E) == 2 ? 2 : 1;   // 32-element k-steps per LDS stage (fp32 panels are twice as large)
     static constexpr int CE = 16 / sizeof(E);       // elements per 16-byte chunk
-    static constexpr int CPR = 32 / CE;              // chunks per 32-element row
-    static constexpr int LD = 32 + CE;               // LDS row stride in elements (16-byte aligned rows, skewed banks)
+    static constexpr int CPR = 32 * KS / CE;         // chunks per staged row
+    static constexpr int LD = 32 * KS + CE;          // LDS row stride in elements (16-byte aligned rows, skewed banks)
 };
 
 __device__ __forceinline__ u32x4 zero_chunk() { return u32x4{0u, 0u, 0u, 0u}; }
@@ -71,7 +72,7 @@ template <typename E, int EPI, int TM, int TN>
 __global__ __launch_bounds__(256) void linear_kernel(pcb_linear_args a) {
     constexpr bool TWO = EPI == PCB_EPI_SILU_MUL;
     constexpr int BM = 32 * TM, BN = 32 * TN, BROWS = TWO ? 2 * BN : BN;
-    constexpr int CE = Tile<E>::CE, CPR = Tile<E>::CPR, LD = Tile<E>::LD;
+    constexpr int CE = Tile<E>::CE, CPR = Tile<E>::CPR, LD = Tile<E>::LD, KS = Tile<E>::KS;
     constexpr int A_CH = (BM * CPR + 255) / 256, B_CH = (BROWS * CPR + 255) / 256;
     __shared__ __attribute__((aligned(16))) E As[BM * LD];
     __shared__ __attribute__((aligned(16))) E Bs[BROWS * LD];
@@ -152,8 +153,8 @@ __global__ __launch_bounds__(256) void linear_kernel(pcb_linear_args a) {
 #pragma unroll
     for (int i = 0; i < B_CH; ++i) rb[i] = load_chunk<E>(b_row[i], b_k[i], K, vec, 1.0f, false);
 
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        __syncthreads();                           // the previous step's fragment reads are done
+    for (int k0 = 0; k0 < K; k0 += 32 * KS) {
+        __syncthreads();                           // the previous stage's fragment reads are done
 #pragma unroll
         for (int i = 0; i < A_CH; ++i)
             if (a_at[i] >= 0) *reinterpret_cast<u32x4*>(&As[a_at[i]]) = ra[i];
@@ -161,24 +162,27 @@ __global__ __launch_bounds__(256) void linear_kernel(pcb_linear_args a) {
         for (int i = 0; i < B_CH; ++i)
             if (b_at[i] >= 0) *reinterpret_cast<u32x4*>(&Bs[b_at[i]]) = rb[i];
         __syncthreads();
-        if (k0 + 32 < K) {
+        if (k0 + 32 * KS < K) {
 #pragma unroll
-            for (int i = 0; i < A_CH; ++i) ra[i] = load_chunk<E>(a_row[i], k0 + 32 + a_k[i], K, vec, a_scale[i], scaled);
+            for (int i = 0; i < A_CH; ++i) ra[i] = load_chunk<E>(a_row[i], k0 + 32 * KS + a_k[i], K, vec, a_scale[i], scaled);
 #pragma unroll
-            for (int i = 0; i < B_CH; ++i) rb[i] = load_chunk<E>(b_row[i], k0 + 32 + b_k[i], K, vec, 1.0f, false);
+            for (int i = 0; i < B_CH; ++i) rb[i] = load_chunk<E>(b_row[i], k0 + 32 * KS + b_k[i], K, vec, 1.0f, false);
         }
-        Frag<E> fa[TM];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = load_frag(&As[((wm * TM + i) * 16 + l15) * LD], group, 32, true);
+        for (int ks = 0; ks < KS; ++ks) {
+            Frag<E> fa[TM];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const Frag<E> fb = load_frag(&Bs[((wn * TN + j) * 16 + l15) * LD], group, 32, true);
+            for (int i = 0; i < TM; ++i) fa[i] = load_frag(&As[((wm * TM + i) * 16 + l15) * LD + 32 * ks], group, 32, true);
 #pragma unroll
-            for (int i = 0; i < TM; ++i) acc[i][j] = mma(fa[i], fb, acc[i][j]);
-            if (TWO) {
-                const Frag<E> fb2 = load_frag(&Bs[(BN + (wn * TN + j) * 16 + l15) * LD], group, 32, true);
+            for (int j = 0; j < TN; ++j) {
+                const Frag<E> fb = load_frag(&Bs[((wn * TN + j) * 16 + l15) * LD + 32 * ks], group, 32, true);
 #pragma unroll
-                for (int i = 0; i < TM; ++i) acc2[i][j] = mma(fa[i], fb2, acc2[i][j]);
+                for (int i = 0; i < TM; ++i) acc[i][j] = mma(fa[i], fb, acc[i][j]);
+                if (TWO) {
+                    const Frag<E> fb2 = load_frag(&Bs[(BN + (wn * TN + j) * 16 + l15) * LD + 32 * ks], group, 32, true);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) acc2[i][j] = mma(fa[i], fb2, acc2[i][j]);
+                }
             }
         }
     }
