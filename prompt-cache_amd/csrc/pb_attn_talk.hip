@@ -18,13 +18,13 @@ struct TileRec {
 };
 
 // ---- 1. scores ---------------------------------------------------------------------------------------------------------------
-// Workgroup = one 16-query tile x KC keys; a wave owns 16-key subtiles of them, one after the other.  The tile's queries (all
+// Workgroup = one 16-query tile x KC keys (128, or 64 when the launch has few tiles: decoding); a wave owns 16-key subtiles of
+// them, one after the other.  The tile's queries (all
 // heads) wait in LDS when they fit (q_lds), so the per-subtile traffic is the keys alone; a key fragment is loaded once per key
 // head and used by every query head of its group.
-constexpr int KC = 128;
 
 template <typename E, int HMAX>
-__global__ __launch_bounds__(256) void talk_scores_kernel(pcb_attn_talk_args a, int band, int q_lds, int qld) {
+__global__ __launch_bounds__(256) void talk_scores_kernel(pcb_attn_talk_args a, int band, int q_lds, int qld, int KC) {
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn[];
     __shared__ __attribute__((aligned(16))) float talk[HMAX * HMAX];      // [h][g], rows padded with zeros
     __shared__ float slope[HMAX];
@@ -296,7 +296,7 @@ __global__ __launch_bounds__(256) void talk_values_few_kernel(pcb_attn_talk_args
         }
         __syncthreads();
         if (active && wide) {
-#pragma unroll 4
+#pragma unroll 16
             for (int kk = slice; kk < n; kk += n_slices) {
                 __attribute__((aligned(16))) E tmp[CE];
                 *reinterpret_cast<u32x4*>(tmp) = *reinterpret_cast<const u32x4*>(V + (int64_t)(j0 + kk) * D + dcol * CE);
@@ -355,8 +355,9 @@ void launch_scores(const pcb_attn_talk_args& a, int band, hipStream_t stream) {
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
         raised = true;
     }
+    const int KC = a.n_tiles >= 64 ? 128 : 64;
     const dim3 grid(a.n_tiles, pcb_ceil_div(band, KC));
-    hipLaunchKernelGGL(kern, grid, dim3(256), q_lds ? q_bytes : 0, stream, a, band, q_lds, qld);
+    hipLaunchKernelGGL(kern, grid, dim3(256), q_lds ? q_bytes : 0, stream, a, band, q_lds, qld, KC);
 }
 
 template <typename E>
