@@ -90,8 +90,11 @@ class KazolornHIP:
                        bqk=torch.cat([e(p + "mix.q.b"), e(p + "mix.k.b")], dim=0).contiguous(),
                        talk=f(p + "mix.talk"), wo=e(p + "mix.o"), bo=e(p + "mix.o.b"),
                        slopes=distance_slopes(l.heads).to(dev))
-            if ent["dwa"].numel() != i + 2:
+            if ent["dwa"].numel() < i + 2:
                 raise ValueError(f"{p}dwa has {ent['dwa'].numel()} weights, layer {i} sums {i + 2} streams")
+            ent["dwa"] = ent["dwa"].reshape(-1)[:i + 2].contiguous()
+            if l.heads > 32 or l.dim > 256:
+                raise ValueError(f"layer {i}: the attention kernels take up to 32 heads of up to 256 columns (got {l.heads} x {l.dim})")
             if l.mlp_kind:
                 ent.update(g2=f(p + "norm2"), ls2=f(p + "ls2"))
             if l.mlp_kind == "dense":

@@ -323,6 +323,8 @@ def load_kazolorn_safetensors(path: str, cfg):
     if missing:
         raise KeyError(f"{path}: tensors missing for this configuration: {missing[:6]}{' ...' if len(missing) > 6 else ''}")
     for k, shp in want.items():
+        if k.endswith(".dwa") and raw[k].dim() == 1 and raw[k].shape[0] >= shp[0]:
+            continue                                  # (a longer table is read up to the streams the layer has)
         if tuple(raw[k].shape) != tuple(shp):
             raise ValueError(f"{path}: {k} has shape {tuple(raw[k].shape)}, the configuration implies {tuple(shp)}")
     return {k: raw[k] for k in want}

@@ -417,6 +417,16 @@ def test_arena_grows_under_a_live_request(dtype):
     assert rel(torch.cat([first, rest]), run_alone(m, t)) < tol(dtype, 1e-6, 1.5e-2)
 
 
+def test_long_prompt_in_several_attention_calls(monkeypatch):
+    """A prompt whose score band would not fit the scratch budget runs its attention over runs of tiles; same logits."""
+    from promptcache_amd.model import kazolorn_hip
+    s, w, m = model("wide", torch.float32)
+    t = toks(150, s.vocab_size, seed=13)
+    whole = run_alone(m, t)
+    monkeypatch.setattr(kazolorn_hip, "ATTN_SCRATCH_FLOATS", 3 * 16 * 16 * 160)      # three 16-row tiles per call
+    assert rel(run_alone(m, t), whole) < 1e-6
+
+
 def test_greedy_generation_through_both_engines():
     from promptcache_amd import BatchEngine, GenerationEngine, GenerationParameters
     from promptcache_amd.model import Kazolorn
