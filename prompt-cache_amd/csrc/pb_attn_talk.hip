@@ -23,7 +23,7 @@ struct TileRec {
 // heads) wait in LDS when they fit (q_lds), so the per-subtile traffic is the keys alone; a key fragment is loaded once per key
 // head and used by every query head of its group.
 
-template <typename E, int HMAX>
+template <typename E, int HMAX, int NST, int PG>
 __global__ __launch_bounds__(256) void talk_scores_kernel(pcb_attn_talk_args a, int band, int q_lds, int qld, int KC) {
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn[];
     __shared__ __attribute__((aligned(16))) float talk[HMAX * HMAX];      // [h][g], rows padded with zeros
@@ -48,12 +48,20 @@ __global__ __launch_bounds__(256) void talk_scores_kernel(pcb_attn_talk_args a, 
     E* Qs = reinterpret_cast<E*>(dyn);
     if (q_lds) {
         if (vec) {
-            const int cpr = HD / 8;
-            for (int e = tid; e < 16 * cpr; e += 256) {
-                const int r = e / cpr, c = (e % cpr) * 8;
-                u32x4 v = u32x4{0u, 0u, 0u, 0u};
-                if (r < t.nq) v = *reinterpret_cast<const u32x4*>(Q + (int64_t)(t.row0 + r) * a.ldq + c);
-                *reinterpret_cast<u32x4*>(Qs + r * qld + c) = v;
+            const int cpr = HD / 8, total = 16 * cpr;
+            for (int e0 = tid; e0 < total; e0 += 256 * 8) {       // eight loads in flight per thread, then their LDS stores
+                u32x4 v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int e = e0 + 256 * u, r = e / cpr, c = (e % cpr) * 8;
+                    v[u] = u32x4{0u, 0u, 0u, 0u};
+                    if (e < total && r < t.nq) v[u] = *reinterpret_cast<const u32x4*>(Q + (int64_t)(t.row0 + r) * a.ldq + c);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int e = e0 + 256 * u, r = e / cpr, c = (e % cpr) * 8;
+                    if (e < total) *reinterpret_cast<u32x4*>(Qs + r * qld + c) = v[u];
+                }
             }
         } else {
             for (int e = tid; e < 16 * HD; e += 256) {
@@ -76,25 +84,38 @@ __global__ __launch_bounds__(256) void talk_scores_kernel(pcb_attn_talk_args a, 
         float s[HMAX][4];
 #pragma unroll
         for (int h = 0; h < HMAX; ++h) s[h][0] = s[h][1] = s[h][2] = s[h][3] = 0.0f;
-        for (int c = 0; c < a.Hkv; ++c) {
-            const E* krow = C + (int64_t)c * a.head_stride + (int64_t)jk * D;
-            Frag<E> fk[8];
+        // the key fragments of PG key heads are requested together (one memory round trip per PG heads, not per head)
+        for (int c0 = 0; c0 < a.Hkv; c0 += PG) {
+            Frag<E> fk[PG][NST];
 #pragma unroll
-            for (int st = 0; st < 8; ++st)
-                if (st < nsteps) fk[st] = load_frag(krow + 32 * st, group, key_ok ? D - 32 * st : 0, vec);
+            for (int u = 0; u < PG; ++u) {
+                const bool ok = key_ok && c0 + u < a.Hkv;
+                const E* krow = C + (int64_t)(ok ? c0 + u : 0) * a.head_stride + (int64_t)(ok ? jk : 0) * D;
+#pragma unroll
+                for (int st = 0; st < NST; ++st)
+                    if (st < nsteps) fk[u][st] = load_frag(krow + 32 * st, group, ok ? D - 32 * st : 0, vec);
+            }
 #pragma unroll
             for (int h = 0; h < HMAX; ++h) {
-                if (h / rep == c && h < H) {
+                const int c = h / rep;
+                if (h < H && c >= c0 && c < c0 + PG) {
                     f4 acc = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int st = 0; st < 8; ++st)
-                        if (st < nsteps) {
-                            const Frag<E> fq = load_frag(qrow0 + h * D + 32 * st, group, q_ok ? D - 32 * st : 0, vec);
-                            acc = mma(fq, fk[st], acc);
+                    for (int u = 0; u < PG; ++u)
+                        if (c - c0 == u) {
+#pragma unroll
+                            for (int st = 0; st < NST; ++st)
+                                if (st < nsteps) {
+                                    const Frag<E> fq = load_frag(qrow0 + h * D + 32 * st, group, q_ok ? D - 32 * st : 0, vec);
+                                    acc = mma(fq, fk[u][st], acc);
+                                }
                         }
                     // lane: key column l15 (j = j0 + l15), query rows 4 * group + r
 #pragma unroll
                     for (int r = 0; r < 4; ++r) s[h][r] = acc[r] * a.scale - slope[h] * (float)(t.q0 + 4 * group + r - jk);
+                    // (a head's query fragments come from LDS and die here: keep the scheduler from hoisting all heads' reads to the
+                    // top of the unrolled loop, which costs the registers of every head at once)
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
@@ -169,32 +190,56 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
 #pragma unroll
     for (int i = 0; i < NP; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
 
-    for (int j0 = j_min; j0 <= i_last; j0 += 32) {
-        for (int e = tid; e < n_sub * 16 * 32; e += 256) {
-            const int r = e >> 5, kk = e & 31;
+    // Software pipeline over 32-key steps: the band values and key chunks of step n + 1 are requested before the MFMAs of step n
+    // and turned into LDS operands after them, so a step costs its arithmetic and two barriers, not a memory round trip.
+    constexpr int SP = 8;                             // band values per thread and step: 64 rows x 32 keys / 256 threads
+    constexpr int VC = NP * (int)sizeof(E) / 8;       // 16-byte key chunks per thread and step: 32 keys x D / CE / 256
+    const int cpk = D / CE;
+    float sv[SP];
+    u32x4 vv[VC];
+    auto fetch = [&](int j0) {
+#pragma unroll
+        for (int u = 0; u < SP; ++u) {
+            const int e = tid + 256 * u, r = e >> 5, kk = e & 31;
             const int dist = t.q0 + r - (j0 + kk);
-            float p = 0.0f;
-            if (r < t.nq && dist >= 0 && dist < window) p = expf(S[r * s_row + dist] - row_m[r]) * row_inv[r];
-            if (SPLIT) {
-                const E hi = from_f32<E>(p);
-                Ph[r * LD + kk] = hi;
-                Pl[r * LD + kk] = from_f32<E>(p - to_f32(hi));
-            } else {
-                Ph[r * LD + kk] = from_f32<E>(p);
+            sv[u] = -INFINITY;
+            if (e < n_sub * 512 && r < t.nq && dist >= 0 && dist < window) sv[u] = S[r * s_row + dist];
+        }
+        if (vec) {
+#pragma unroll
+            for (int u = 0; u < VC; ++u) {
+                const int e = tid + 256 * u, kk = e & 31, c = (e >> 5) * CE;
+                vv[u] = u32x4{0u, 0u, 0u, 0u};
+                if (e < 32 * cpk && j0 + kk <= i_last) vv[u] = *reinterpret_cast<const u32x4*>(V + (int64_t)(j0 + kk) * D + c);
+            }
+        }
+    };
+    fetch(j_min);
+    for (int j0 = j_min; j0 <= i_last; j0 += 32) {
+#pragma unroll
+        for (int u = 0; u < SP; ++u) {
+            const int e = tid + 256 * u, r = e >> 5, kk = e & 31;
+            if (e < n_sub * 512) {
+                const float p = sv[u] == -INFINITY ? 0.0f : expf(sv[u] - row_m[r]) * row_inv[r];
+                if (SPLIT) {
+                    const E hi = from_f32<E>(p);
+                    Ph[r * LD + kk] = hi;
+                    Pl[r * LD + kk] = from_f32<E>(p - to_f32(hi));
+                } else {
+                    Ph[r * LD + kk] = from_f32<E>(p);
+                }
             }
         }
         if (vec) {
-            const int cpk = D / CE;                   // 16-byte chunks per key
-            for (int e = tid; e < 32 * cpk; e += 256) {
-                const int kk = e & 31, c = (e >> 5) * CE;
-                const int j = j0 + kk;
-                __attribute__((aligned(16))) E tmp[CE];
-                if (j <= i_last)
-                    *reinterpret_cast<u32x4*>(tmp) = *reinterpret_cast<const u32x4*>(V + (int64_t)j * D + c);
-                else
-                    *reinterpret_cast<u32x4*>(tmp) = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-                for (int i = 0; i < CE; ++i) Vt[(c + i) * LD + kk] = tmp[i];
+            for (int u = 0; u < VC; ++u) {
+                const int e = tid + 256 * u, kk = e & 31, c = (e >> 5) * CE;
+                if (e < 32 * cpk) {
+                    __attribute__((aligned(16))) E tmp[CE];
+                    *reinterpret_cast<u32x4*>(tmp) = vv[u];
+#pragma unroll
+                    for (int i = 0; i < CE; ++i) Vt[(c + i) * LD + kk] = tmp[i];
+                }
             }
             for (int e = tid; e < 32 * (D16 - D); e += 256) Vt[(D + e / 32) * LD + (e & 31)] = from_f32<E>(0.0f);
         } else {
@@ -205,6 +250,7 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
             }
         }
         __syncthreads();
+        if (j0 + 32 <= i_last) fetch(j0 + 32);
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
             const int p = wave + 4 * i;
@@ -349,11 +395,14 @@ void launch_scores(const pcb_attn_talk_args& a, int band, hipStream_t stream) {
     const size_t q_bytes = (size_t)16 * qld * sizeof(E);
     const bool aligned = (a.H * a.head_dim) % ce == 0;
     const int q_lds = aligned && q_bytes + sizeof(float) * (HMAX * HMAX + HMAX) <= 150 * 1024;
-    auto kern = talk_scores_kernel<E, HMAX>;
-    static bool raised = false;
-    if (q_lds && q_bytes > 48 * 1024 && !raised) {
+    // NST = k-steps of a head (head_dim / 32, rounded up) the kernel is built for, PG = key heads fetched together
+    constexpr int PG = (HMAX <= 16 && sizeof(E) == 2) ? 4 : 2;
+    auto kern = a.head_dim <= 128 ? talk_scores_kernel<E, HMAX, 4, PG> : talk_scores_kernel<E, HMAX, 8, (PG > 2 ? 2 : PG)>;
+    static bool raised[2] = {false, false};
+    bool& up = raised[a.head_dim <= 128 ? 0 : 1];
+    if (q_lds && q_bytes > 48 * 1024 && !up) {
         hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-        raised = true;
+        up = true;
     }
     const int KC = a.n_tiles >= 64 ? 128 : 64;
     const dim3 grid(a.n_tiles, pcb_ceil_div(band, KC));

@@ -3,7 +3,7 @@
 //
 // Every kernel is a template over the element type E of weights, activations and cached keys: `bf16_t` (matrix products on
 // v_mfma_f32_16x16x32_bf16, fp32 accumulation) or `float` (v_mfma_f32_16x16x4_f32: true fp32 products).  One "k-step" is 32
-// contraction elements in both cases, so the tiling code does not branch on the type.
+// k elements in both cases, so the tiling code does not branch on the type.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
@@ -83,7 +83,7 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // ---- MFMA operand fragments of one 32-element k-step -----------------------------------------------------------------
 // A 16 x 32 operand tile (16 rows of the A matrix, or 16 columns of B given as rows of B^T) is held by a wave as: lane l owns
-// row (l & 15) and the 8 contraction elements lane_k<E>(l >> 4, e), e = 0..7.  bf16: 8 consecutive elements (one MFMA);
+// row (l & 15) and the 8 k elements lane_k<E>(l >> 4, e), e = 0..7.  bf16: 8 consecutive elements (one MFMA);
 // fp32: elements 4*e + group (eight 16x16x4 MFMAs).  A and B use the same map, so any k permutation cancels.
 template <typename E>
 struct Frag;
@@ -107,7 +107,7 @@ __device__ __forceinline__ int lane_k<float>(int group, int e) {
     return 4 * e + group;
 }
 
-// p points at contraction element 0 of this k-step in the lane's row; `valid` elements from there exist (<= 0: none).
+// p points at k element 0 of this k-step in the lane's row; `valid` elements from there exist (<= 0: none).
 // `vec`: p + 8*group is 16-byte aligned and the row may be read with one 16-byte load (bf16 only).
 __device__ __forceinline__ Frag<bf16_t> load_frag(const bf16_t* p, int group, int valid, bool vec) {
     Frag<bf16_t> f;

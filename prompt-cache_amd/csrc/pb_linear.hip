@@ -20,7 +20,7 @@ struct Tile {
 
 __device__ __forceinline__ u32x4 zero_chunk() { return u32x4{0u, 0u, 0u, 0u}; }
 
-// one 16-byte chunk of row `p` (null: a row outside the matrix) starting at contraction element k, K elements in the row
+// one 16-byte chunk of row `p` (null: a row outside the matrix) starting at k element k, K elements in the row
 template <typename E>
 __device__ __forceinline__ u32x4 load_chunk(const E* p, int k, int K, bool vec, float scale, bool scaled) {
     constexpr int CE = Tile<E>::CE;
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void linear_kernel(pcb_linear_args a) {
 }
 
 // ---- few rows: the weights stream once, straight from memory into the matrix cores --------------------------------------------
-// Workgroup = 16 result columns x up to 16 rows; its eight waves split the contraction (k-step s goes to wave s % 8) and add their
+// Workgroup = 16 result columns x up to 16 rows; its eight waves split the k range (k-step s goes to wave s % 8) and add their
 // partial tiles through LDS.  No LDS staging: a lane's B fragment is 16 contiguous bytes of its weight row, its A fragment 16
 // bytes of its activation row (a handful of rows that stay in cache).
 template <typename E>

@@ -1502,7 +1502,7 @@ def test_shared_prefix_attention_equals_the_prefix_copied_into_every_row(prefix_
 def test_dense_qkv_rope_epilogue_equals_projection_then_rope_append(B, q_len, H, Hkv, two, ragged):
     """pc_gemm_dense_qkv_rope (RoPE + KV append in the epilogue of the many-row q|k|v projection, head_dim 128) against the two
     launches it replaces: pc_gemm_dense (fp32 [M][W]) + pc_rope_append.  Same fp32 accumulators, same rotation formula:
-    identical bits for V and for every row the arena does not touch, fp32 round-off (an fma contraction) at most elsewhere."""
+    identical bits for V and for every row the arena does not touch, fp32 round-off (an fma inner-dimension) at most elsewhere."""
     n = _n()
     rng = np.random.default_rng(17 + q_len)
     D, K = 128, 256
