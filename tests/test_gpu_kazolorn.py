@@ -266,6 +266,11 @@ def _attn_case(dtype, H, G, D, window, n, first, talk_noise=0.2, seed=0, spike=N
     (16, 4, 32, 70, 200, 0),     # many heads, window across key blocks
     (3, 3, 6, 4, 19, 17),        # two rows ending a sequence
     (32, 8, 8, 33, 50, 0),       # the most heads the kernel takes
+    (12, 4, 24, 0, 70, 0),       # head counts between the kernel's register tiers
+    (24, 24, 16, 21, 45, 40),
+    (2, 1, 160, 40, 90, 0),      # heads wider than 128 columns (the 8-step score kernel, 16 value subtiles)
+    (4, 2, 256, 0, 37, 30),      # ... and the widest
+    (20, 5, 136, 17, 40, 0),     # many heads AND wide heads
 ])
 def test_attention_alone(dtype, H, G, D, window, n, first):
     got, want, _ = _attn_case(dtype, H, G, D, window, n, first)
@@ -307,7 +312,7 @@ def test_attention_sink_and_mixing_matter():
 # the model through its arena
 # =====================================================================================================================================
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,n", [("mixed", 45), ("odd", 19), ("wide", 150)])
+@pytest.mark.parametrize("name,n", [("mixed", 45), ("odd", 19), ("wide", 150), ("wide", 330)])      # 330: > 64 rows per expert
 def test_prompt_matches_oracle_layer_by_layer(name, n, dtype):
     s, w, m = model(name, dtype)
     t = toks(n, s.vocab_size, seed=1)
@@ -402,6 +407,16 @@ def test_same_rows_same_values_whatever_the_company():
     assert rel(both, alone) < 1e-6
     other = m.forward_rows(ar, [s1], [a], [list(range(21))])              # same row count, another slot, dirty neighbours
     assert torch.equal(other, alone)
+    # one-token steps (captured graph): logits of the rows that ask for them only, whatever the others ask for
+    nxt_a, nxt_b = 5, 9
+    full = m.forward_rows(ar, [s0, s2], [[nxt_a], [nxt_b]], [[0], [0]])
+    ar2 = m.new_arena(2, 64)
+    t0, t1 = ar2.alloc(), ar2.alloc()
+    m.forward_rows(ar2, [t0, t1], [a, b], [[], []])
+    part = m.forward_rows(ar2, [t0, t1], [[nxt_a], [nxt_b]], [[], [0]])
+    none = m.forward_rows(ar2, [t0, t1], [[1], [2]], [[], []])
+    assert part.shape == (1, s.vocab_size) and none.shape == (0, s.vocab_size)
+    assert rel(part, full[1:2]) < 1e-6
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
