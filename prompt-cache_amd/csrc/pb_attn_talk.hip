@@ -288,7 +288,7 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
 // A row's output is a weighted sum of key rows: no matrix core needed, and nothing to transpose.  Thread = (column d, key slice);
 // it walks its slice's keys with coalesced loads (a key row is contiguous over d), multiplies by the rows' weights from LDS
 // (fp32, not rounded) and the slices meet in LDS at the end.
-constexpr int FEW_ROWS = 4, FEW_KEYS = 512;
+constexpr int FEW_ROWS = 4, FEW_KEYS = 1024;
 
 template <typename E>
 __global__ __launch_bounds__(256) void talk_values_few_kernel(pcb_attn_talk_args a, int band, const int32_t* tiles) {
@@ -304,19 +304,35 @@ __global__ __launch_bounds__(256) void talk_values_few_kernel(pcb_attn_talk_args
     const int j_min = t.q0 - window + 1 > 0 ? t.q0 - window + 1 : 0;
     const float* __restrict__ S = a.scratch + ((int64_t)t.row0 * H + h) * band;
     const int64_t s_row = (int64_t)H * band;
-    for (int r = wave; r < t.nq; r += 4) {
+    // row statistics in one pass, all threads on one row at a time: a thread folds its share of the row into a (max, sum) pair
+    // -- every load of the row is in flight at once -- and the pairs meet in LDS
+    for (int r = 0; r < t.nq; ++r) {
         const int i = t.q0 + r;
         const int n = i + 1 < window ? i + 1 : window;
         const float* sr = S + r * s_row;
-        float m = a.sink ? 0.0f : -INFINITY;
-        for (int d = lane; d < n; d += 64) m = fmaxf(m, sr[d]);
-        m = wave_max(m);
-        float l = 0.0f;
-        for (int d = lane; d < n; d += 64) l += expf(sr[d] - m);
-        l = wave_sum(l);
-        if (a.sink) l += expf(-m);
-        if (lane == 0) row_m[r] = m, row_inv[r] = 1.0f / l;
+        float m = -INFINITY, l = 0.0f;
+        for (int d = tid; d < n; d += 256) {
+            const float v = sr[d];
+            const float m2 = fmaxf(m, v);
+            l = l * expf(m - m2) + expf(v - m2);
+            m = m2;
+        }
+        const float wm = wave_max(m);
+        l = wave_sum(m == -INFINITY ? 0.0f : l * expf(m - wm));
+        if (lane == 0) red[0][wave] = wm, red[1][wave] = l;
+        __syncthreads();
+        if (tid == 0) {
+            float bm = a.sink ? 0.0f : -INFINITY;
+            for (int w = 0; w < 4; ++w) bm = fmaxf(bm, red[0][w]);
+            float bl = a.sink ? expf(-bm) : 0.0f;
+            for (int w = 0; w < 4; ++w)
+                if (red[0][w] != -INFINITY) bl += red[1][w] * expf(red[0][w] - bm);
+            row_m[r] = bm;
+            row_inv[r] = 1.0f / bl;
+        }
+        __syncthreads();
     }
+    for (int e = tid; e < FEW_ROWS * FEW_KEYS; e += 256) (&P[0][0])[e] = 0.0f;      // rows the tile does not have stay zero
     __syncthreads();
     const E* __restrict__ V = (const E*)a.cache + (int64_t)t.slot * a.slot_stride + (int64_t)(h / rep) * a.head_stride;
     // wide form: a thread owns one 16-byte chunk of the key rows (CE columns) and every (256 / chunks)-th key
@@ -333,11 +349,11 @@ __global__ __launch_bounds__(256) void talk_values_few_kernel(pcb_attn_talk_args
         for (int i = 0; i < CE; ++i) acc[r][i] = 0.0f;
     for (int j0 = j_min; j0 <= i_last; j0 += FEW_KEYS) {
         const int n = i_last - j0 + 1 < FEW_KEYS ? i_last - j0 + 1 : FEW_KEYS;
-        for (int e = tid; e < FEW_ROWS * FEW_KEYS; e += 256) {
+        for (int e = tid; e < t.nq * FEW_KEYS; e += 256) {
             const int r = e / FEW_KEYS, kk = e % FEW_KEYS;
             const int dist = t.q0 + r - (j0 + kk);
             float p = 0.0f;
-            if (r < t.nq && kk < n && dist >= 0 && dist < window) p = expf(S[r * s_row + dist] - row_m[r]) * row_inv[r];
+            if (kk < n && dist >= 0 && dist < window) p = expf(S[r * s_row + dist] - row_m[r]) * row_inv[r];
             P[r][kk] = p;
         }
         __syncthreads();
