@@ -143,6 +143,8 @@ class KazolornHIP:
         counts = [len(t) for t in tokens]
         if len(set(slots)) != len(slots) or len(slots) != len(tokens):
             raise ValueError("one distinct slot per request")
+        if not counts:
+            return torch.empty((0, self.V), dtype=f32, device=dev)
         if min(counts, default=1) < 1:
             raise ValueError("every request of a step brings at least one token")
         T = sum(counts)
