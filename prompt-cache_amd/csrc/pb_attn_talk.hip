@@ -145,15 +145,15 @@ __global__ __launch_bounds__(256) void talk_scores_kernel(pcb_attn_talk_args a, 
 }
 
 // ---- 2. values ---------------------------------------------------------------------------------------------------------------
-// Workgroup = up to 64 consecutive queries of one sequence (a tile of the second table) x one head.  Row statistics first; then
-// per 32 keys: the rows' weights into LDS (hi + lo for bf16), the keys transposed into LDS once for all rows, and the
-// (16-row subtile, 16-column subtile) products dealt round-robin to the four waves.
+// Workgroup = up to 64 consecutive queries of one sequence (a tile of the second table) x one head.  Per 32 keys: the rows'
+// unnormalised weights into LDS (hi + lo for bf16) with a running maximum / denominator per row, the keys transposed into LDS
+// once for all rows, and the (16-row subtile, 16-column subtile) products dealt round-robin to the four waves.
 template <typename E, int NP>
 __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, int band, const int32_t* tiles) {
     constexpr bool SPLIT = sizeof(E) == 2;           // bf16: P as hi + lo
     constexpr int CE = 16 / sizeof(E), LD = 32 + CE;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    __shared__ float row_m[64], row_inv[64];
+    __shared__ float row_alpha[64], row_inv[64];
     __shared__ __attribute__((aligned(16))) E Ph[64 * LD];
     __shared__ __attribute__((aligned(16))) E Pl[SPLIT ? 64 * LD : 1];
     E* Vt = reinterpret_cast<E*>(lds_raw);           // [D16][LD]: Vt[d][key]
@@ -169,21 +169,6 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
     const int64_t s_row = (int64_t)H * band;
     const int n_sub = (t.nq + 15) / 16, n_dt = D16 / 16, n_pairs = n_sub * n_dt;
 
-    for (int r = wave; r < t.nq; r += 4) {
-        const int i = t.q0 + r;
-        const int n = i + 1 < window ? i + 1 : window;
-        const float* sr = S + r * s_row;
-        float m = a.sink ? 0.0f : -INFINITY;
-        for (int d = lane; d < n; d += 64) m = fmaxf(m, sr[d]);
-        m = wave_max(m);
-        float l = 0.0f;
-        for (int d = lane; d < n; d += 64) l += expf(sr[d] - m);
-        l = wave_sum(l);
-        if (a.sink) l += expf(-m);
-        if (lane == 0) row_m[r] = m, row_inv[r] = 1.0f / l;
-    }
-    __syncthreads();
-
     const E* V = (const E*)a.cache + (int64_t)t.slot * a.slot_stride + (int64_t)(h / rep) * a.head_stride;
     const bool vec = D % CE == 0 && a.head_stride % CE == 0 && a.slot_stride % CE == 0 && ((uintptr_t)a.cache % 16 == 0);
     f4 acc[NP];
@@ -192,53 +177,96 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
 
     // Software pipeline over 32-key steps: the band values and key chunks of step n + 1 are requested before the MFMAs of step n
     // and turned into LDS operands after them, so a step costs its arithmetic and two barriers, not a memory round trip.
+    // A thread owns 4 consecutive keys of a row (twice: rows r and r + 32) and the same 16-byte column chunk of 2 consecutive
+    // keys, so its LDS operands go out as 8- and 4-byte stores (4 + 8 per step and thread) instead of one per element.
     constexpr int SP = 8;                             // band values per thread and step: 64 rows x 32 keys / 256 threads
-    constexpr int VC = NP * (int)sizeof(E) / 8;       // 16-byte key chunks per thread and step: 32 keys x D / CE / 256
+    constexpr int VC = NP * (int)sizeof(E) / 8 < 2 ? 2 : NP * (int)sizeof(E) / 8;     // 16-byte key chunks per thread and step (in pairs)
     const int cpk = D / CE;
     float sv[SP];
     u32x4 vv[VC];
     auto fetch = [&](int j0) {
 #pragma unroll
-        for (int u = 0; u < SP; ++u) {
-            const int e = tid + 256 * u, r = e >> 5, kk = e & 31;
-            const int dist = t.q0 + r - (j0 + kk);
-            sv[u] = -INFINITY;
-            if (e < n_sub * 512 && r < t.nq && dist >= 0 && dist < window) sv[u] = S[r * s_row + dist];
+        for (int u = 0; u < SP / 4; ++u) {
+            const int e = tid + 256 * u, r = e >> 3, kq = (e & 7) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int dist = t.q0 + r - (j0 + kq + i);
+                sv[4 * u + i] = -INFINITY;
+                if (r < n_sub * 16 && r < t.nq && dist >= 0 && dist < window) sv[4 * u + i] = S[r * s_row + dist];
+            }
         }
         if (vec) {
 #pragma unroll
             for (int u = 0; u < VC; ++u) {
-                const int e = tid + 256 * u, kk = e & 31, c = (e >> 5) * CE;
+                // chunk index within the step: pair p of keys (2p, 2p + 1), column chunk c; u even: key 2p, u odd: key 2p + 1
+                const int pe = tid + 256 * (u >> 1), kk = (pe & 15) * 2 + (u & 1), c = (pe >> 4) * CE;
                 vv[u] = u32x4{0u, 0u, 0u, 0u};
-                if (e < 32 * cpk && j0 + kk <= i_last) vv[u] = *reinterpret_cast<const u32x4*>(V + (int64_t)(j0 + kk) * D + c);
+                if (pe < 16 * cpk && j0 + kk <= i_last) vv[u] = *reinterpret_cast<const u32x4*>(V + (int64_t)(j0 + kk) * D + c);
             }
         }
     };
+    // Online softmax: the 8 lanes that own a row's 32 keys of a step keep its running maximum and denominator (the sink enters
+    // as maximum 0, denominator 1), publish the factor that rescales what the row has accumulated so far, and write unnormalised
+    // weights; the division by the denominator happens once, at the end.  The band is read exactly once.
+    float rm[SP / 4], rl[SP / 4];
+#pragma unroll
+    for (int u = 0; u < SP / 4; ++u) rm[u] = a.sink ? 0.0f : -INFINITY, rl[u] = a.sink ? 1.0f : 0.0f;
     fetch(j_min);
     for (int j0 = j_min; j0 <= i_last; j0 += 32) {
 #pragma unroll
-        for (int u = 0; u < SP; ++u) {
-            const int e = tid + 256 * u, r = e >> 5, kk = e & 31;
-            if (e < n_sub * 512) {
-                const float p = sv[u] == -INFINITY ? 0.0f : expf(sv[u] - row_m[r]) * row_inv[r];
+        for (int u = 0; u < SP / 4; ++u) {
+            const int e = tid + 256 * u, r = e >> 3, kq = (e & 7) * 4;
+            float tmax = fmaxf(fmaxf(sv[4 * u], sv[4 * u + 1]), fmaxf(sv[4 * u + 2], sv[4 * u + 3]));
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 1, 64));
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 2, 64));
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 4, 64));
+            const float m_new = fmaxf(rm[u], tmax);
+            const float alpha = m_new == -INFINITY ? 1.0f : expf(rm[u] - m_new);
+            float pv[4], psum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pv[i] = sv[4 * u + i] == -INFINITY ? 0.0f : expf(sv[4 * u + i] - m_new);
+                psum += pv[i];
+            }
+            psum += __shfl_xor(psum, 1, 64);
+            psum += __shfl_xor(psum, 2, 64);
+            psum += __shfl_xor(psum, 4, 64);
+            rl[u] = rl[u] * alpha + psum;
+            rm[u] = m_new;
+            if (r < n_sub * 16) {
+                if ((lane & 7) == 0) row_alpha[r] = alpha;
+                __attribute__((aligned(16))) E hi[4];
+                __attribute__((aligned(16))) E lo[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    hi[i] = from_f32<E>(pv[i]);
+                    if (SPLIT) lo[i] = from_f32<E>(pv[i] - to_f32(hi[i]));
+                }
                 if (SPLIT) {
-                    const E hi = from_f32<E>(p);
-                    Ph[r * LD + kk] = hi;
-                    Pl[r * LD + kk] = from_f32<E>(p - to_f32(hi));
+                    *reinterpret_cast<uint64_t*>(&Ph[r * LD + kq]) = *reinterpret_cast<const uint64_t*>(hi);
+                    *reinterpret_cast<uint64_t*>(&Pl[r * LD + kq]) = *reinterpret_cast<const uint64_t*>(lo);
                 } else {
-                    Ph[r * LD + kk] = from_f32<E>(p);
+                    *reinterpret_cast<u32x4*>(&Ph[r * LD + kq]) = *reinterpret_cast<const u32x4*>(hi);
                 }
             }
         }
         if (vec) {
 #pragma unroll
-            for (int u = 0; u < VC; ++u) {
-                const int e = tid + 256 * u, kk = e & 31, c = (e >> 5) * CE;
-                if (e < 32 * cpk) {
-                    __attribute__((aligned(16))) E tmp[CE];
-                    *reinterpret_cast<u32x4*>(tmp) = vv[u];
+            for (int u = 0; u < VC; u += 2) {
+                const int pe = tid + 256 * (u >> 1), kk = (pe & 15) * 2, c = (pe >> 4) * CE;
+                if (pe < 16 * cpk) {
+                    __attribute__((aligned(16))) E t0[CE];
+                    __attribute__((aligned(16))) E t1[CE];
+                    *reinterpret_cast<u32x4*>(t0) = vv[u];
+                    *reinterpret_cast<u32x4*>(t1) = vv[u + 1];
 #pragma unroll
-                    for (int i = 0; i < CE; ++i) Vt[(c + i) * LD + kk] = tmp[i];
+                    for (int i = 0; i < CE; ++i) {
+                        __attribute__((aligned(8))) E pr[2] = {t0[i], t1[i]};
+                        if (sizeof(E) == 2)
+                            *reinterpret_cast<uint32_t*>(&Vt[(c + i) * LD + kk]) = *reinterpret_cast<const uint32_t*>(pr);
+                        else
+                            *reinterpret_cast<uint64_t*>(&Vt[(c + i) * LD + kk]) = *reinterpret_cast<const uint64_t*>(pr);
+                    }
                 }
             }
             for (int e = tid; e < 32 * (D16 - D); e += 256) Vt[(D + e / 32) * LD + (e & 31)] = from_f32<E>(0.0f);
@@ -258,6 +286,8 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
                 const int sub = p % n_sub, dt = p / n_sub;
                 const Frag<E> ph = load_frag(&Ph[(sub * 16 + l15) * LD], group, 32, true);
                 const Frag<E> fv = load_frag(&Vt[(dt * 16 + l15) * LD], group, 32, true);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[i][r] *= row_alpha[sub * 16 + 4 * group + r];
                 acc[i] = mma(ph, fv, acc[i]);
                 if (SPLIT) {
                     const Frag<E> pl = load_frag(&Pl[(sub * 16 + l15) * LD], group, 32, true);
@@ -267,6 +297,12 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
         }
         __syncthreads();
     }
+#pragma unroll
+    for (int u = 0; u < SP / 4; ++u) {
+        const int r = (tid + 256 * u) >> 3;
+        if ((lane & 7) == 0) row_inv[r] = 1.0f / rl[u];
+    }
+    __syncthreads();
     E* O = (E*)a.out;
 #pragma unroll
     for (int i = 0; i < NP; ++i) {
@@ -277,7 +313,7 @@ __global__ __launch_bounds__(256) void talk_values_kernel(pcb_attn_talk_args a, 
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int qr = sub * 16 + 4 * group + r;
-                    if (qr < t.nq) O[(int64_t)(t.row0 + qr) * a.ldo + h * D + d] = from_f32<E>(acc[i][r]);
+                    if (qr < t.nq) O[(int64_t)(t.row0 + qr) * a.ldo + h * D + d] = from_f32<E>(acc[i][r] * row_inv[qr]);
                 }
             }
         }
