@@ -6,8 +6,10 @@
 //      MFMA result layout a lane then holds the same four (query, key) pairs of all heads, so bias, mixing
 //      (H x H fp32 multiply-adds per pair) and the window test are lane-local.  The mixed scores go to an fp32 band
 //      [row][head][distance i - j] -- no softmax state, hence no coupling between key tiles: the grid runs over key blocks too.
-//   2. talk_values_kernel: per (query tile, head): row maximum and denominator from the band (the sink enters as a score of 0),
-//      then P V on the matrix cores with the keys as values; bf16 runs P as a hi + lo pair so the fp32 weights are not rounded.
+//   2. talk_values_kernel: per (up to 64 queries, head): one sweep over the band with a running maximum and denominator per row
+//      (the sink enters as a score of 0), P V on the matrix cores with the keys as values; bf16 runs P as a hi + lo pair so the
+//      fp32 weights are not rounded.  Tiles of at most 4 rows (decoding) take talk_values_few_kernel: fp32 multiply-adds over
+//      coalesced key rows, no matrix cores.
 #include "pb_common.h"
 
 namespace {
