@@ -295,10 +295,174 @@ class KazolornShape:
         return cls(vocab_size=vocab, hidden_size=width, norm_eps=eps, layers=layers, name=name)
 
 
+@dataclass
+class DibizenLayer:
+    """One layer of a Dibizen stack.  ``kind``: which mixer it has --
+
+    * ``"lightning"``: linear attention with one scalar decay per head (``decay``), ``heads`` heads of ``dim`` query/key and
+      ``vdim`` value columns;
+    * ``"attention"``: causal softmax attention, ``heads`` query heads over ``kv_heads`` key/value heads, scores scaled by
+      ``scale``, queries scaled by a temperature that grows with the logarithm of the position (``qt_coef``, ``qt_every``;
+      ``qt_every`` 0 = none), ``kv_from`` >= 0: no key/value projections of its own, it reads that layer's cache;
+    * ``"mamba1"``: selective scan over ``inner`` channels with ``state`` states each, a causal convolution of ``conv`` taps in
+      front, step sizes through a ``dt_rank``-wide bottleneck.
+
+    The feed-forward (``experts`` 0 = none) is a mixture of ``experts`` squared-ReLU experts of width ``ff`` plus ``identity``
+    experts that return their input; ``top`` of them are chosen per token among the best ``groups_keep`` of ``groups`` groups."""
+    kind: str
+    heads: int = 0
+    kv_heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    scale: float = 1.0
+    decay: tuple = ()
+    qt_coef: float = 0.0
+    qt_every: int = 0
+    kv_from: int = -1
+    inner: int = 0
+    state: int = 0
+    conv: int = 0
+    dt_rank: int = 0
+    ff: int = 0
+    experts: int = 0
+    identity: int = 0
+    top: int = 0
+    groups: int = 1
+    groups_keep: int = 1
+
+
+@dataclass
+class DibizenShape:
+    """Dibizen: decoder-only, learned absolute positions, ``streams`` residual streams mixed by hyper-connections around every
+    sublayer, Dynamic-Tanh norms, layers whose mixer is lightning (decayed linear) attention, gated softmax attention (which may
+    borrow an earlier layer's keys and values) or a Mamba selective scan, mixture-of-experts feed-forwards with a corrected,
+    group-limited softmax router and identity experts, and soft-capped logits.  Every size and constant comes from
+    ``config.json`` (``from_config``); layers may differ from one another and come in any order."""
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: list
+    streams: int = 1
+    max_positions: int = 0
+    logit_softcap: float = 0.0
+    name: str = "dibizen"
+
+    ARCHITECTURE = "Dibizen"
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_config(cls, c: dict, name: str = "dibizen") -> "DibizenShape":
+        if c.get("architecture") != cls.ARCHITECTURE:
+            raise ValueError(f"config.json describes {c.get('architecture')!r}, not {cls.ARCHITECTURE}")
+        layers = []
+        for i, lc in enumerate(c["layers"]):
+            kind, m = lc.get("type"), lc.get("mixer") or {}
+            if kind == "lightning":
+                lay = DibizenLayer(kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                                   decay=tuple(float(d) for d in m["decay"]))
+                lay.kv_heads = lay.heads
+                if len(lay.decay) != lay.heads:
+                    raise ValueError(f"layer {i}: {len(lay.decay)} decays for {lay.heads} heads")
+            elif kind == "attention":
+                heads, dim = int(m["heads"]), int(m["dim"])
+                kv = int(m.get("kv_heads", heads))
+                if heads % kv:
+                    raise ValueError(f"layer {i}: {heads} query heads do not divide over {kv} key heads")
+                qt = m.get("q_temp") or {}
+                lay = DibizenLayer(kind, heads=heads, kv_heads=kv, dim=dim, vdim=int(m.get("vdim", dim)),
+                                   scale=float(m.get("scale", dim ** -0.5)), qt_coef=float(qt.get("coef", 0.0)),
+                                   qt_every=int(qt.get("every", 0)) if qt else 0,
+                                   kv_from=int(m["kv_from"]) if m.get("kv_from") is not None else -1)
+                if lay.kv_from >= 0:
+                    src = layers[lay.kv_from] if lay.kv_from < i else None
+                    if src is None or src.kind != "attention" or src.kv_from >= 0 or \
+                            (src.kv_heads, src.dim, src.vdim) != (lay.kv_heads, lay.dim, lay.vdim):
+                        raise ValueError(f"layer {i}: kv_from {lay.kv_from} must name an earlier attention layer with projections "
+                                         f"of its own and the same key/value heads and sizes")
+            elif kind == "mamba1":
+                lay = DibizenLayer(kind, inner=int(m["inner"]), state=int(m["state"]), conv=int(m["conv"]), dt_rank=int(m["dt_rank"]))
+                if lay.conv < 1:
+                    raise ValueError(f"layer {i}: a convolution has at least one tap")
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+            mlp = lc.get("mlp")
+            if mlp:
+                if mlp.get("kind", "moe") != "moe":
+                    raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+                r = mlp["router"]
+                g = r.get("groups") or {}
+                lay.ff, lay.experts, lay.identity = int(mlp["expert"]["ff"]), int(r["experts"]), int(r.get("identity", 0))
+                lay.top, lay.groups = int(r["top"]), int(g.get("count", 1))
+                lay.groups_keep = int(g.get("keep", lay.groups))
+                total = lay.experts + lay.identity
+                if total % lay.groups or not 1 <= lay.groups_keep <= lay.groups:
+                    raise ValueError(f"layer {i}: {total} router outputs in {lay.groups} groups, {lay.groups_keep} kept")
+                if not 1 <= lay.top <= total // lay.groups * lay.groups_keep:
+                    raise ValueError(f"layer {i}: top {lay.top} of {total} router outputs with {lay.groups_keep} of {lay.groups} groups")
+            layers.append(lay)
+        return cls(vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), norm_eps=float((c.get("norm") or {}).get("eps", 1e-5)),
+                   layers=layers, streams=int(c.get("streams", 1)), max_positions=int(c["max_positions"]),
+                   logit_softcap=float(c.get("logit_softcap") or 0.0), name=name)
+
+    @classmethod
+    def from_dir(cls, path: str) -> "DibizenShape":
+        with open(os.path.join(path, "config.json")) as f:
+            return cls.from_config(json.load(f), name=os.path.basename(os.path.normpath(path)))
+
+    def to_config(self) -> dict:
+        """The ``config.json`` form (what ``from_config`` reads)."""
+        out = []
+        for l in self.layers:
+            if l.kind == "lightning":
+                mixer = {"decay": list(l.decay), "dim": l.dim, "heads": l.heads, "vdim": l.vdim}
+            elif l.kind == "attention":
+                mixer = {"dim": l.dim, "heads": l.heads, "kv_heads": l.kv_heads, "scale": l.scale, "vdim": l.vdim}
+                if l.qt_every:
+                    mixer["q_temp"] = {"coef": l.qt_coef, "every": l.qt_every}
+                if l.kv_from >= 0:
+                    mixer["kv_from"] = l.kv_from
+            else:
+                mixer = {"conv": l.conv, "dt_rank": l.dt_rank, "inner": l.inner, "state": l.state}
+            mlp = None
+            if l.experts + l.identity:
+                mlp = {"kind": "moe", "expert": {"ff": l.ff},
+                       "router": {"experts": l.experts, "groups": {"count": l.groups, "keep": l.groups_keep},
+                                  "identity": l.identity, "top": l.top}}
+            out.append({"type": l.kind, "mixer": mixer, "mlp": mlp})
+        return {"architecture": self.ARCHITECTURE, "layers": out, "logit_softcap": self.logit_softcap,
+                "max_positions": self.max_positions, "norm": {"eps": self.norm_eps}, "streams": self.streams,
+                "vocab": self.vocab_size, "width": self.hidden_size}
+
+    @classmethod
+    def uniform(cls, vocab: int, width: int, pattern, heads: int, kv_heads: int, dim: int, experts: int, top: int, expert_ff: int,
+                identity: int = 0, groups: int = 1, groups_keep: int = 1, streams: int = 2, inner: int = 0, state: int = 16,
+                max_positions: int = 8192, name: str = "dibizen") -> "DibizenShape":
+        """A stack whose layers follow ``pattern`` (a sequence of mixer kinds), all with the same sizes and feed-forward."""
+        layers = []
+        for kind in pattern:
+            if kind == "lightning":
+                lay = DibizenLayer(kind, heads=heads, kv_heads=heads, dim=dim, vdim=dim,
+                                   decay=tuple(1.0 - 2.0 ** (-5.0 - 3.0 * h / max(1, heads - 1)) for h in range(heads)))
+            elif kind == "attention":
+                lay = DibizenLayer(kind, heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, qt_coef=0.1,
+                                   qt_every=1024)
+            else:
+                lay = DibizenLayer("mamba1", inner=inner or 2 * width, state=state, conv=4, dt_rank=max(1, width // 16))
+            lay.ff, lay.experts, lay.identity, lay.top, lay.groups, lay.groups_keep = expert_ff, experts, identity, top, groups, groups_keep
+            layers.append(lay)
+        return cls(vocab_size=vocab, hidden_size=width, norm_eps=1e-5, layers=layers, streams=streams, max_positions=max_positions,
+                   logit_softcap=30.0, name=name)
+
+
 def architecture_of(path: str) -> str:
     """Which model family a checkpoint directory holds: ``architecture`` (Kazolorn) or HF's ``model_type``."""
     with open(os.path.join(path, "config.json")) as f:
         c = json.load(f)
     if c.get("architecture") == KazolornShape.ARCHITECTURE:
         return "kazolorn"
+    if c.get("architecture") == DibizenShape.ARCHITECTURE:
+        return "dibizen"
     return str(c.get("model_type", "llama"))
