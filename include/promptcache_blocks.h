@@ -16,7 +16,7 @@
 extern "C" {
 #endif
 
-#define PCB_ABI_VERSION 1
+#define PCB_ABI_VERSION 2
 #define PCB_OK 0
 #define PCB_ERR_ARG (-2001)
 #define PCB_ERR_HIP_BASE (-3000)
@@ -68,6 +68,13 @@ int pcb_mix_norm(const pcb_mix_norm_args* a, void* stream);
 #define PCB_EPI_STORE 0
 #define PCB_EPI_SILU_MUL 1
 #define PCB_EPI_SCALE_ADD 2
+/* element-wise function of a STORE epilogue: z, z sigmoid(z), sigmoid(z), max(z, 0)^2, ln(1 + e^z), cap tanh(z / cap) */
+#define PCB_ACT_NONE 0
+#define PCB_ACT_SILU 1
+#define PCB_ACT_SIGMOID 2
+#define PCB_ACT_RELU2 3
+#define PCB_ACT_SOFTPLUS 4
+#define PCB_ACT_SOFTCAP 5
 typedef struct pcb_linear_args {
     uint32_t struct_bytes;
     int32_t dtype;
@@ -96,6 +103,10 @@ typedef struct pcb_linear_args {
     const int64_t* row_off2;
     int32_t head_dim2;
     int64_t head_stride2;
+    int32_t act;       /* PCB_ACT_*: STORE only, applied to acc + bias before the store (not to the columns split off to y2) */
+    int32_t act_split; /* > 0: columns n >= act_split take act2 instead of act */
+    int32_t act2;
+    float act_param;   /* PCB_ACT_SOFTCAP: the cap */
 } pcb_linear_args;
 int pcb_linear(const pcb_linear_args* a, void* stream);
 
@@ -154,6 +165,162 @@ typedef struct pcb_attn_talk_args {
 } pcb_attn_talk_args;
 int32_t pcb_attn_talk_band(int32_t window, int32_t max_kv_len);
 int pcb_attn_talk(const pcb_attn_talk_args* a, void* stream);
+
+/* ---- residual streams, norms, routers of designs with several residual streams --------------------------------------------- */
+
+/* out[s][r][:] = fp32(table[ids[r]]) + fp32(pos_table[positions[r]]) for every stream s < n_streams (pos_table null: no
+ * position term).  out is fp32 [n_streams][.. stream_stride ..]. */
+int pcb_embed_pos_rows(const void* table, const void* pos_table, int32_t dtype, const int32_t* ids, const int32_t* positions,
+                       float* out, int64_t stream_stride, int32_t n_streams, int32_t n_rows, int32_t width, int32_t vocab,
+                       int32_t max_positions, void* stream);
+
+/* Hyper-connection step around a sublayer, one workgroup per row, in two optional halves:
+ *   write (y given):   x_t <- sum_s mix[s][t] x_s + out_w[t] * y[src]        all streams t at once from the old ones, in place
+ *                      (with `rows` the new streams are used but not written back)
+ *   read (out given):  u = sum_s in_w[s] x_s  (in_w null: the plain sum),  out[r] = norm(u) as E,  x_out[r] = u (fp32) if given
+ * norm: PCB_NORM_NONE u; PCB_NORM_RMS u / sqrt(mean(u^2) + eps) * gain; PCB_NORM_DYT tanh(alpha[0] * u) * gain + bias.
+ * src = rows ? rows[r] : r.  n_streams <= 8. */
+#define PCB_NORM_NONE 0
+#define PCB_NORM_RMS 1
+#define PCB_NORM_DYT 2
+typedef struct pcb_hyper_norm_args {
+    uint32_t struct_bytes;
+    int32_t dtype;
+    float* streams;
+    int64_t stream_stride;
+    int32_t n_streams;
+    const float* y; /* fp32 [rows][width] */
+    const float* mix;   /* [S][S], indexed [from][to] */
+    const float* out_w; /* [S] */
+    const float* in_w;  /* [S] or null */
+    int32_t norm;
+    const float* gain;
+    const float* bias;
+    const float* alpha; /* one float on the device */
+    float eps;
+    void* out;
+    float* x_out;
+    const int32_t* rows;
+    int32_t n_rows;
+    int32_t width;
+} pcb_hyper_norm_args;
+int pcb_hyper_norm(const pcb_hyper_norm_args* a, void* stream);
+
+/* out[r][c] = E( (gain ? x[r][c] / sqrt(mean_c x[r]^2 + eps) * gain[c] : x[r][c]) * (gate ? gate[r][c] : 1) ), x fp32 [n_rows][ldx],
+ * gate E [n_rows][ldg], out E [n_rows][ldo]: a unit norm over all heads' outputs with an element-wise gate. */
+int pcb_gated_norm(const float* x, int64_t ldx, const float* gain, const void* gate, int64_t ldg, void* out, int64_t ldo,
+                   int32_t dtype, float eps, int32_t n_rows, int32_t cols, void* stream);
+
+/* Router choice over n_out outputs per row (logits fp32 [n_rows][n_out]):
+ *   score s = score_fn == PCB_SCORE_SOFTMAX ? softmax(logits) : sigmoid(logits);  choice score = s + correction (if given)
+ *   groups > 1: outputs form `groups` equal runs of neighbours; a group's score is its largest choice score; only outputs of
+ *   the groups_keep best groups can be chosen
+ *   the `top` largest choice scores win (ties: the lower index); weight = s (without the correction), divided by the sum of
+ *   the chosen weights + 1e-20 when renorm.  pair p = r * top + k: expert[p], weight[p].  n_out <= 2048, groups <= 64. */
+#define PCB_SCORE_SIGMOID 0
+#define PCB_SCORE_SOFTMAX 1
+int pcb_router_select(const float* logits, int32_t n_rows, int32_t n_out, int32_t top, int32_t score_fn, const float* correction,
+                      int32_t groups, int32_t groups_keep, int32_t renorm, int32_t* expert, float* weight, void* stream);
+
+/* y[r][:] = sum_k weight[p] * (expert[p] >= n_real ? h[r][:] : pair_out[p][:]),  p = r * top + k  (fixed order over k):
+ * the weighted sum of a token's experts' results, identity experts (index >= n_real) standing for the token's own input h
+ * (E [n_rows][width]).  y fp32 [n_rows][width] is overwritten. */
+int pcb_moe_mix(const float* pair_out, const int32_t* expert, const float* weight, const void* h, int32_t dtype, int32_t n_real,
+                float* y, int32_t n_rows, int32_t width, int32_t top, void* stream);
+
+/* ---- mixers ------------------------------------------------------------------------------------------------------------------- */
+
+/* Causal softmax attention over a slot-addressed cache with separate keys and values.
+ * Queries are flat rows; tile t = {slot, first query position, query rows (<= 16), first flat row} (int32 x 4, device).
+ * Key j of kv head g of slot s: kcache + s * slot_stride + g * head_stride + j * row_stride (dim elements); its value at the same
+ * offset from vcache (vdim elements) -- keys and values may interleave in one plane.  The cache already holds the queries' own
+ * keys.  score = q_scale[row] * scale * q.k (q_scale null: 1); key j is seen by the query at position i iff j <= i and
+ * (window <= 0 or i - j < window).  The result (E [rows][ldo], head h at column h * vdim) is multiplied element-wise by
+ * gate[row][..] (E, ldg) when given.  dim, vdim <= 256. */
+typedef struct pcb_attn_softmax_args {
+    uint32_t struct_bytes;
+    int32_t dtype;
+    const void* q;
+    int64_t ldq;
+    const float* q_scale;
+    const int32_t* tiles;
+    int32_t n_tiles;
+    const void* kcache;
+    const void* vcache;
+    int64_t slot_stride, head_stride, row_stride;
+    int32_t H, Hkv, dim, vdim;
+    float scale;
+    int32_t window;
+    const void* gate;
+    int64_t ldg;
+    void* out;
+    int64_t ldo;
+} pcb_attn_softmax_args;
+int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream);
+
+/* Linear attention with one scalar decay per head and a matrix state per (slot, head):
+ *   S_t = decay[h] * S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t        (S: [dim][vdim], fp32, zero before position 0)
+ * q, k: E rows with head h at column h * dim; v: head h at column h * vdim; out fp32 [rows][ldo].  request r = {slot, first
+ * position, tokens, first flat row} (int32 x 4, device): its tokens are consecutive rows; a request that starts at position 0
+ * starts from a zero state whatever the slot held.  state: fp32 [slots][H][dim][vdim] (slot_stride floats per slot), read at the
+ * start and written at the end of each request.  All products run on the fp32 matrix cores.  dim <= 256. */
+typedef struct pcb_decay_attn_args {
+    uint32_t struct_bytes;
+    int32_t dtype;
+    const void* q;
+    const void* k;
+    const void* v;
+    int64_t ldq, ldk, ldv;
+    const int32_t* reqs;
+    int32_t n_reqs;
+    float* state;
+    int64_t slot_stride;
+    const float* decay;
+    int32_t H, dim, vdim;
+    float* out;
+    int64_t ldo;
+} pcb_decay_attn_args;
+int pcb_decay_attn(const pcb_decay_attn_args* a, void* stream);
+
+/* Causal per-channel convolution of `taps` taps (the last tap is the current token's) with bias and optional SiLU:
+ *   out[r][c] = act( bias[c] + sum_j w[c][j] * in(pos(r) - (taps - 1) + j)[c] ),  in(p) = 0 for p < 0
+ * row_meta[r] = {slot, position, index of the row among its request's rows of this step, 0}: inputs older than the step come from
+ * state (E [slots][taps - 1][C]: the last taps - 1 inputs of the slot).  pcb_conv_state_update then moves the state behind the
+ * step's rows (reqs as in pcb_decay_attn); it must run after pcb_causal_conv of the same step.  taps <= 16. */
+int pcb_causal_conv(const void* x, int64_t ldx, const void* w, const void* bias, int32_t dtype, int32_t silu, const int32_t* row_meta,
+                    const void* state, int64_t slot_stride, void* out, int64_t ldo, int32_t n_rows, int32_t C, int32_t taps,
+                    void* stream);
+int pcb_conv_state_update(const void* x, int64_t ldx, int32_t dtype, const int32_t* reqs, int32_t n_reqs, void* state,
+                          int64_t slot_stride, int32_t C, int32_t taps, void* stream);
+
+/* Selective scan (one state vector of N floats per channel):
+ *   S[c][n] <- exp(dt[c] * A[c][n]) * S[c][n] + dt[c] * x[c] * B[n],   y[c] = sum_n S[c][n] * Cm[n] + D[c] * x[c],
+ *   out[c] = y[c] * silu(z[c])   (z null: out = y)
+ * per token, in order, for each request {slot, first position, tokens, first flat row}.  x, z: E rows; dt, B, Cm: fp32 rows;
+ * A fp32 [C][N], D fp32 [C]; state fp32 [slots][C][N] (zero before position 0); out E.  N <= 256. */
+typedef struct pcb_selective_scan_args {
+    uint32_t struct_bytes;
+    int32_t dtype;
+    const void* x;
+    int64_t ldx;
+    const float* dt;
+    int64_t lddt;
+    const float* B;
+    const float* Cm;
+    int64_t ldbc;
+    const void* z;
+    int64_t ldz;
+    const float* A;
+    const float* D;
+    const int32_t* reqs;
+    int32_t n_reqs;
+    float* state;
+    int64_t slot_stride;
+    int32_t C, N;
+    void* out;
+    int64_t ldo;
+} pcb_selective_scan_args;
+int pcb_selective_scan(const pcb_selective_scan_args* a, void* stream);
 
 #ifdef __cplusplus
 }

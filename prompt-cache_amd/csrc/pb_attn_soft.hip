@@ -1,0 +1,233 @@
+// pcb_attn_softmax: causal softmax attention over a slot-addressed cache with separate keys and values (grouped key/value
+// heads, value size independent of the key size, optional sliding window, per-row score factor, optional output gate).
+//
+// One workgroup = one tile of up to 16 queries x one query head; its four waves take every fourth block of 32 keys and keep a
+// running maximum / denominator per query (online softmax), then merge through LDS.  Both products are "swapped" so that no
+// operand is transposed between them:
+//   S^T = K Q^T   a wave's result tile has the query in the lane's column (l & 15) and keys 4 (l >> 4) + r in its rows,
+//   O^T = V^T P^T the weights P of a query are exactly what its lanes hold; the k index of this product runs over the 32 keys of
+//                 the block in the order (l >> 4, e) -> key 4 (l >> 4) + e (e < 4), 16 + 4 (l >> 4) + e - 4 (e >= 4), the same for
+//                 both operands, so the permutation cancels.
+// Scores, maxima, weights and sums are fp32.  bf16: the weights enter the second product as a hi + lo pair of bf16 values (two
+// MFMAs), so they are not rounded to 8 bits; fp32: the fp32 matrix cores take them as they are.
+#include "pb_common.h"
+
+namespace {
+using namespace pcb;
+
+constexpr int AW = 4;          // waves of a workgroup
+
+template <typename E>
+struct PFrag;
+template <>
+struct PFrag<bf16_t> {
+    Frag<bf16_t> hi, lo;
+};
+template <>
+struct PFrag<float> {
+    Frag<float> hi;
+};
+
+__device__ __forceinline__ void make_p(PFrag<bf16_t>& f, const float (&p)[8]) {
+    uint32_t h[8], l[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        h[e] = bf16_bits(p[e]);
+        l[e] = bf16_bits(p[e] - __uint_as_float(h[e] << 16));
+    }
+    f.hi.v = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+    f.lo.v = u32x4{l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16)};
+}
+__device__ __forceinline__ void make_p(PFrag<float>& f, const float (&p)[8]) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f.hi.v[e] = p[e];
+}
+
+// the value operand of one 16-column block: element e of lane (column c, group g) is V[key(g, e)][c]
+__device__ __forceinline__ Frag<bf16_t> load_v(const bf16_t* const (&rows)[8], int c, bool ok) {
+    Frag<bf16_t> f;
+    uint32_t w[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) w[e] = ok ? rows[e][c].bits : 0u;
+    f.v = u32x4{w[0] | (w[1] << 16), w[2] | (w[3] << 16), w[4] | (w[5] << 16), w[6] | (w[7] << 16)};
+    return f;
+}
+__device__ __forceinline__ Frag<float> load_v(const float* const (&rows)[8], int c, bool ok) {
+    Frag<float> f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f.v[e] = ok ? rows[e][c] : 0.0f;
+    return f;
+}
+
+__device__ __forceinline__ f4 mma_p(const Frag<bf16_t>& v, const PFrag<bf16_t>& p, f4 c) {
+    c = mma(v, p.hi, c);
+    return mma(v, p.lo, c);
+}
+__device__ __forceinline__ f4 mma_p(const Frag<float>& v, const PFrag<float>& p, f4 c) { return mma(v, p.hi, c); }
+
+// KSQ: 32-element k-steps of the key size; VB: 16-column blocks of the value size
+template <typename E, int KSQ, int VB>
+__global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_args a) {
+    __shared__ float red_o[AW - 1][VB * 256];
+    __shared__ float red_ml[AW - 1][2][16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, c = lane & 15;
+    const int32_t* tile = a.tiles + 4 * blockIdx.x;
+    const int slot = tile[0], pos0 = tile[1], rows = tile[2], row0 = tile[3];
+    const int h = blockIdx.y, hk = h / (a.H / a.Hkv);
+    const int dim = a.dim, vdim = a.vdim;
+    const int last = pos0 + rows - 1;                       // the newest key any query of the tile sees
+    const int qi = c < rows ? c : rows - 1;                 // (lanes past the tile repeat its last query; nothing of theirs is stored)
+    const int qpos = pos0 + qi;
+    const int64_t qrow = row0 + qi;
+    const E* K = (const E*)a.kcache + (int64_t)slot * a.slot_stride + (int64_t)hk * a.head_stride;
+    const E* V = (const E*)a.vcache + (int64_t)slot * a.slot_stride + (int64_t)hk * a.head_stride;
+    const E* qp = (const E*)a.q + qrow * a.ldq + (int64_t)h * dim;
+    constexpr int CE = 16 / sizeof(E);
+    const bool qvec = ((uintptr_t)a.q % 16 == 0) && (a.ldq % CE == 0) && (dim % CE == 0);
+    const bool kvec = ((uintptr_t)a.kcache % 16 == 0) && (a.slot_stride % CE == 0) && (a.head_stride % CE == 0) && (a.row_stride % CE == 0);
+    Frag<E> qf[KSQ];
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ++ks) qf[ks] = load_frag(qp + 32 * ks, g, dim - 32 * ks, qvec);
+    const float sc = a.scale * (a.q_scale ? a.q_scale[qrow] : 1.0f);
+    const float NEG = -__builtin_inff();
+
+    float m = NEG, l = 0.0f;
+    f4 o[VB];
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb) o[vb] = f4{0.f, 0.f, 0.f, 0.f};
+
+    const int kb_lo = a.window > 0 ? (pos0 - a.window + 1 > 0 ? (pos0 - a.window + 1) / 32 : 0) : 0;
+    const int kb_hi = last / 32;
+    for (int kb = kb_lo + wave; kb <= kb_hi; kb += AW) {
+        float s[8];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            int j = kb * 32 + kt * 16 + c;                  // this lane's key row of the K operand
+            j = j > last ? last : j;
+            const E* kp = K + (int64_t)j * a.row_stride;
+            f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KSQ; ++ks) acc = mma(load_frag(kp + 32 * ks, g, dim - 32 * ks, kvec), qf[ks], acc);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = kb * 32 + kt * 16 + 4 * g + r;
+                const bool seen = key <= qpos && (a.window <= 0 || qpos - key < a.window);
+                s[kt * 4 + r] = seen ? acc[r] * sc : NEG;
+            }
+        }
+        float bm = s[0];
+#pragma unroll
+        for (int e = 1; e < 8; ++e) bm = fmaxf(bm, s[e]);
+        bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+        bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+        const float m_new = fmaxf(m, bm);
+        const float m_use = m_new == NEG ? 0.0f : m_new;
+        const float alpha = expf(m - m_use);                // (m = -inf: 0)
+        float p[8], psum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            p[e] = expf(s[e] - m_use);
+            psum += p[e];
+        }
+        l = l * alpha + psum;
+        m = m_new;
+        PFrag<E> pf;
+        make_p(pf, p);
+        const E* vrows[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            int key = kb * 32 + (e < 4 ? 4 * g + e : 16 + 4 * g + e - 4);
+            key = key > last ? last : key;
+            vrows[e] = V + (int64_t)key * a.row_stride;
+        }
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb) {
+            if (vb * 16 >= vdim) break;
+            const int col = vb * 16 + c;
+            const Frag<E> vf = load_v(vrows, col, col < vdim);
+            f4 t = o[vb];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) t[r] *= alpha;
+            o[vb] = mma_p(vf, pf, t);
+        }
+    }
+    // the denominator's parts of the four lane groups
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+
+    // merge the waves: wave 0 collects
+    if (wave > 0) {
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red_o[wave - 1][(vb * 4 + r) * 64 + lane] = o[vb][r];
+        if (g == 0) {
+            red_ml[wave - 1][0][c] = m;
+            red_ml[wave - 1][1][c] = l;
+        }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    float mm = m;
+#pragma unroll
+    for (int w = 0; w < AW - 1; ++w) mm = fmaxf(mm, red_ml[w][0][c]);
+    const float m_use = mm == NEG ? 0.0f : mm;
+    float f0 = expf(m - m_use);
+    float lt = l * f0;
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[vb][r] *= f0;
+#pragma unroll
+    for (int w = 0; w < AW - 1; ++w) {
+        const float fw = expf(red_ml[w][0][c] - m_use);
+        lt += red_ml[w][1][c] * fw;
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[vb][r] += fw * red_o[w][(vb * 4 + r) * 64 + lane];
+    }
+    if (c >= rows) return;
+    const float inv = 1.0f / lt;
+    E* op = (E*)a.out + qrow * a.ldo + (int64_t)h * vdim;
+    const E* gp = a.gate ? (const E*)a.gate + qrow * a.ldg + (int64_t)h * vdim : nullptr;
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int col = vb * 16 + 4 * g + r;
+            if (col < vdim) {
+                float v = o[vb][r] * inv;
+                if (gp) v *= to_f32(gp[col]);
+                op[col] = from_f32<E>(v);
+            }
+        }
+}
+
+template <typename E>
+int dispatch(const pcb_attn_softmax_args& a, hipStream_t stream) {
+    const dim3 grid(a.n_tiles, a.H), block(64 * AW);
+    const int big = a.dim > a.vdim ? a.dim : a.vdim;
+    if (big <= 64)
+        hipLaunchKernelGGL((attn_softmax_kernel<E, 2, 4>), grid, block, 0, stream, a);
+    else if (big <= 128)
+        hipLaunchKernelGGL((attn_softmax_kernel<E, 4, 8>), grid, block, 0, stream, a);
+    else
+        hipLaunchKernelGGL((attn_softmax_kernel<E, 8, 16>), grid, block, 0, stream, a);
+    return pcb_check_launch("attn_softmax_kernel");
+}
+
+}  // namespace
+
+PCB_EXPORT int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream) {
+    PCB_REQUIRE(a && a->struct_bytes == sizeof(pcb_attn_softmax_args), PCB_ERR_ARG, "pcb_attn_softmax: struct size mismatch");
+    PCB_REQUIRE(a->dtype == PCB_BF16 || a->dtype == PCB_F32, PCB_ERR_ARG, "pcb_attn_softmax: unknown dtype");
+    PCB_REQUIRE(a->n_tiles >= 0 && a->H > 0 && a->Hkv > 0 && a->H % a->Hkv == 0 && a->dim > 0 && a->dim <= 256 && a->vdim > 0 &&
+                    a->vdim <= 256 && a->ldq >= (int64_t)a->H * a->dim && a->ldo >= (int64_t)a->H * a->vdim &&
+                    a->row_stride >= a->dim && a->row_stride >= a->vdim,
+                PCB_ERR_ARG, "pcb_attn_softmax: bad sizes (key and value sizes up to 256)");
+    if (a->n_tiles == 0) return PCB_OK;
+    PCB_REQUIRE(a->q && a->tiles && a->kcache && a->vcache && a->out && (!a->gate || a->ldg >= (int64_t)a->H * a->vdim), PCB_ERR_ARG,
+                "pcb_attn_softmax: null pointer");
+    return a->dtype == PCB_BF16 ? dispatch<pcb::bf16_t>(*a, (hipStream_t)stream) : dispatch<float>(*a, (hipStream_t)stream);
+}

@@ -44,10 +44,23 @@ __device__ __forceinline__ u32x4 load_chunk(const E* p, int k, int K, bool vec, 
     return c;
 }
 
+__device__ __forceinline__ float apply_act(int act, float v, float param) {
+    switch (act) {
+        case PCB_ACT_SILU: return v / (1.0f + expf(-v));
+        case PCB_ACT_SIGMOID: return 1.0f / (1.0f + expf(-v));
+        case PCB_ACT_RELU2: return v > 0.0f ? v * v : 0.0f;
+        case PCB_ACT_SOFTPLUS: return v > 20.0f ? v : log1pf(expf(v));
+        case PCB_ACT_SOFTCAP: return param * tanhf(v / param);
+        default: return v;
+    }
+}
+
 // one result element through the epilogue (see pcb_linear_args)
 template <typename E, int EPI>
 __device__ __forceinline__ void emit(const pcb_linear_args& a, int m, int n, float acc, float acc2, float bv, float cs) {
     float v = acc + bv;
+    if (EPI == PCB_EPI_STORE && (a.act | a.act2) && !(a.split_n > 0 && n >= a.split_n))      // (the split-off part is stored as it is)
+        v = apply_act((a.act_split > 0 && n >= a.act_split) ? a.act2 : a.act, v, a.act_param);
     if (EPI == PCB_EPI_SILU_MUL) v = acc / (1.0f + expf(-acc)) * acc2;
     if (EPI == PCB_EPI_SCALE_ADD) {
         float* y = (float*)a.y + (int64_t)m * a.ldy + n;
@@ -347,6 +360,11 @@ PCB_EXPORT int pcb_linear(const pcb_linear_args* a, void* stream) {
     PCB_REQUIRE(a->dtype == PCB_BF16 || a->dtype == PCB_F32, PCB_ERR_ARG, "pcb_linear: unknown dtype");
     PCB_REQUIRE(a->M >= 0 && a->N > 0 && a->K > 0 && a->ldx >= a->K && a->ldw >= a->K, PCB_ERR_ARG, "pcb_linear: bad sizes");
     PCB_REQUIRE(a->epilogue >= PCB_EPI_STORE && a->epilogue <= PCB_EPI_SCALE_ADD, PCB_ERR_ARG, "pcb_linear: unknown epilogue");
+    PCB_REQUIRE(a->act >= PCB_ACT_NONE && a->act <= PCB_ACT_SOFTCAP && a->act2 >= PCB_ACT_NONE && a->act2 <= PCB_ACT_SOFTCAP &&
+                    a->act_split >= 0 && ((a->act | a->act2) == 0 || a->epilogue == PCB_EPI_STORE),
+                PCB_ERR_ARG, "pcb_linear: an activation goes with the plain store epilogue");
+    PCB_REQUIRE((a->act != PCB_ACT_SOFTCAP && a->act2 != PCB_ACT_SOFTCAP) || a->act_param > 0.0f, PCB_ERR_ARG,
+                "pcb_linear: the soft cap must be positive");
     if (a->M == 0) return PCB_OK;
     PCB_REQUIRE(a->x && a->w && a->y, PCB_ERR_ARG, "pcb_linear: null pointer");
     PCB_REQUIRE(a->n_groups >= 0 && (a->n_groups == 0 || a->group_off), PCB_ERR_ARG, "pcb_linear: groups need their offsets");

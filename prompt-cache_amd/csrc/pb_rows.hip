@@ -258,3 +258,303 @@ PCB_EXPORT int pcb_moe_combine(const float* pair_out, const float* col_scale, fl
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, pair_out, col_scale, y, width, top);
     return pcb_check_launch("moe_combine_kernel");
 }
+
+// ---- several residual streams: embedding with positions, hyper-connection steps with their norms, gated unit norm ----------------
+namespace {
+using namespace pcb;
+
+template <typename E>
+__global__ __launch_bounds__(256) void embed_pos_rows_kernel(const E* __restrict__ table, const E* __restrict__ pos_table,
+                                                             const int32_t* __restrict__ ids, const int32_t* __restrict__ positions,
+                                                             float* __restrict__ out, int64_t stream_stride, int n_streams, int width,
+                                                             int vocab, int max_positions) {
+    const int r = blockIdx.x;
+    int id = ids[r];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const E* src = table + (int64_t)id * width;
+    const E* ps = nullptr;
+    if (pos_table) {
+        int p = positions[r];
+        p = p < 0 ? 0 : (p >= max_positions ? max_positions - 1 : p);
+        ps = pos_table + (int64_t)p * width;
+    }
+    for (int c = threadIdx.x; c < width; c += 256) {
+        const float v = to_f32(src[c]) + (ps ? to_f32(ps[c]) : 0.0f);
+        for (int s = 0; s < n_streams; ++s) out[s * stream_stride + (int64_t)r * width + c] = v;
+    }
+}
+
+constexpr int MAX_STREAMS = 8;
+
+template <typename E>
+__global__ __launch_bounds__(256) void hyper_norm_kernel(pcb_hyper_norm_args a) {
+    extern __shared__ float row[];          // RMS only: the row between the sum and the norm
+    __shared__ float red[16];
+    __shared__ float coef[MAX_STREAMS * MAX_STREAMS + 2 * MAX_STREAMS];
+    const int r = blockIdx.x, S = a.n_streams, W = a.width;
+    const int64_t src = a.rows ? a.rows[r] : r;
+    float* mixw = coef;
+    float* outw = coef + MAX_STREAMS * MAX_STREAMS;
+    float* inw = outw + MAX_STREAMS;
+    if (threadIdx.x < S * S) mixw[threadIdx.x] = a.y ? a.mix[threadIdx.x] : 0.0f;
+    if (threadIdx.x < S) {
+        outw[threadIdx.x] = a.y ? a.out_w[threadIdx.x] : 0.0f;
+        inw[threadIdx.x] = a.in_w ? a.in_w[threadIdx.x] : 1.0f;
+    }
+    __syncthreads();
+    const bool reads = a.out != nullptr || a.x_out != nullptr;
+    const float alpha = a.norm == PCB_NORM_DYT ? a.alpha[0] : 0.0f;
+    float ss[1] = {0.0f};
+    E* o = (E*)a.out;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float x[MAX_STREAMS];
+#pragma unroll
+        for (int s = 0; s < MAX_STREAMS; ++s) x[s] = s < S ? a.streams[s * a.stream_stride + src * W + c] : 0.0f;
+        if (a.y) {
+            const float yv = a.y[src * W + c];
+            float nx[MAX_STREAMS];
+#pragma unroll
+            for (int t = 0; t < MAX_STREAMS; ++t) {
+                float v = 0.0f;
+#pragma unroll
+                for (int s = 0; s < MAX_STREAMS; ++s)
+                    if (s < S && t < S) v += mixw[s * S + t] * x[s];
+                nx[t] = v + (t < S ? outw[t] : 0.0f) * yv;
+            }
+#pragma unroll
+            for (int t = 0; t < MAX_STREAMS; ++t) {
+                x[t] = nx[t];
+                if (t < S && !a.rows) a.streams[t * a.stream_stride + src * W + c] = nx[t];
+            }
+        }
+        if (!reads) continue;
+        float u = 0.0f;
+#pragma unroll
+        for (int s = 0; s < MAX_STREAMS; ++s)
+            if (s < S) u += inw[s] * x[s];
+        if (a.x_out) a.x_out[(int64_t)r * W + c] = u;
+        if (!o) continue;
+        if (a.norm == PCB_NORM_RMS) {
+            row[c] = u;
+            ss[0] += u * u;
+        } else if (a.norm == PCB_NORM_DYT) {
+            o[(int64_t)r * W + c] = from_f32<E>(tanhf(alpha * u) * a.gain[c] + (a.bias ? a.bias[c] : 0.0f));
+        } else {
+            o[(int64_t)r * W + c] = from_f32<E>(u);
+        }
+    }
+    if (o && a.norm == PCB_NORM_RMS) {
+        block_sum<1>(ss, red);
+        const float inv = 1.0f / sqrtf(ss[0] / (float)W + a.eps);
+        for (int c = threadIdx.x; c < W; c += 256) o[(int64_t)r * W + c] = from_f32<E>(row[c] * inv * a.gain[c]);
+    }
+}
+
+template <typename E>
+__global__ __launch_bounds__(256) void gated_norm_kernel(const float* __restrict__ x, int64_t ldx, const float* __restrict__ gain,
+                                                         const E* __restrict__ gate, int64_t ldg, E* __restrict__ out, int64_t ldo,
+                                                         float eps, int cols) {
+    __shared__ float red[16];
+    const int64_t r = blockIdx.x;
+    float ss[1] = {0.0f};
+    float inv = 1.0f;
+    if (gain) {
+        for (int c = threadIdx.x; c < cols; c += 256) {
+            const float v = x[r * ldx + c];
+            ss[0] += v * v;
+        }
+        block_sum<1>(ss, red);
+        inv = 1.0f / sqrtf(ss[0] / (float)cols + eps);
+    }
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        float v = x[r * ldx + c];
+        if (gain) v = v * inv * gain[c];
+        if (gate) v *= to_f32(gate[r * ldg + c]);
+        out[r * ldo + c] = from_f32<E>(v);
+    }
+}
+
+// one wave per row: scores and choice scores in LDS, group maxima by lanes, then rounds of a wave-wide arg-max
+__global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, int n_rows, int n_out, int top, int score_fn,
+                                                            const float* __restrict__ correction, int groups, int keep, int renorm,
+                                                            int32_t* __restrict__ expert, float* __restrict__ weight) {
+    extern __shared__ float sc[];          // per wave: [n_out] scores, [n_out] choice scores, [64] group scores
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = blockIdx.x * 4 + wave;
+    if (r >= n_rows) return;
+    float* s = sc + wave * (2 * n_out + 64);
+    float* ch = s + n_out;
+    float* gs = ch + n_out;
+    const float* z = logits + (int64_t)r * n_out;
+    const float NEG = -__builtin_inff();
+    auto sync = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    if (score_fn == PCB_SCORE_SOFTMAX) {
+        float m = NEG;
+        for (int e = lane; e < n_out; e += 64) m = fmaxf(m, z[e]);
+        m = wave_max(m);
+        float sum = 0.0f;
+        for (int e = lane; e < n_out; e += 64) {
+            const float v = expf(z[e] - m);
+            s[e] = v;
+            sum += v;
+        }
+        sum = wave_sum(sum);
+        for (int e = lane; e < n_out; e += 64) s[e] = s[e] / sum;
+    } else {
+        for (int e = lane; e < n_out; e += 64) s[e] = 1.0f / (1.0f + expf(-z[e]));
+    }
+    for (int e = lane; e < n_out; e += 64) ch[e] = s[e] + (correction ? correction[e] : 0.0f);
+    sync();
+    if (groups > 1) {
+        const int per = n_out / groups;
+        if (lane < groups) {
+            float b = NEG;
+            for (int e = lane * per; e < (lane + 1) * per; ++e) b = fmaxf(b, ch[e]);
+            gs[lane] = b;
+        }
+        sync();
+        // the `keep` best groups stay; the others' choice scores become minus infinity
+        float mine = lane < groups ? gs[lane] : NEG;
+        bool kept = false;
+        for (int k = 0; k < keep; ++k) {
+            float best = (lane < groups && !kept) ? mine : NEG;
+            int bi = (lane < groups && !kept) ? lane : 0x7fffffff;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ov = __shfl_xor(best, o, 64);
+                const int oi = __shfl_xor(bi, o, 64);
+                if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) best = ov, bi = oi;
+            }
+            if (lane == bi) kept = true;
+        }
+        if (lane < groups && !kept)
+            for (int e = lane * per; e < (lane + 1) * per; ++e) ch[e] = NEG;
+        sync();
+    }
+    float wsum = 0.0f;
+    for (int k = 0; k < top; ++k) {
+        float best = NEG;
+        int bi = 0x7fffffff;
+        for (int e = lane; e < n_out; e += 64) {
+            const float v = ch[e];
+            if (v != v) continue;                   // (a taken output is marked with a NaN)
+            if (bi == 0x7fffffff || v > best) best = v, bi = e;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) best = ov, bi = oi;
+        }
+        const float w = s[bi];
+        wsum += w;
+        if (lane == 0) {
+            expert[(int64_t)r * top + k] = bi;
+            weight[(int64_t)r * top + k] = w;
+            ch[bi] = __builtin_nanf("");
+        }
+        sync();
+    }
+    if (renorm && lane < top) weight[(int64_t)r * top + lane] = weight[(int64_t)r * top + lane] / (wsum + 1e-20f);
+}
+
+template <typename E>
+__global__ __launch_bounds__(256) void moe_mix_kernel(const float* __restrict__ pair_out, const int32_t* __restrict__ expert,
+                                                      const float* __restrict__ weight, const E* __restrict__ h, int n_real,
+                                                      float* __restrict__ y, int width, int top) {
+    const int64_t r = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float s = 0.0f;
+        for (int k = 0; k < top; ++k) {
+            const int64_t p = r * top + k;
+            const float v = expert[p] >= n_real ? to_f32(h[r * width + c]) : pair_out[p * width + c];
+            s += weight[p] * v;
+        }
+        y[r * width + c] = s;
+    }
+}
+
+}  // namespace
+
+PCB_EXPORT int pcb_embed_pos_rows(const void* table, const void* pos_table, int32_t dtype, const int32_t* ids, const int32_t* positions,
+                                  float* out, int64_t stream_stride, int32_t n_streams, int32_t n_rows, int32_t width, int32_t vocab,
+                                  int32_t max_positions, void* stream) {
+    PCB_REQUIRE(PCB_DTYPE_OK(dtype) && n_rows >= 0 && width > 0 && vocab > 0 && n_streams >= 1, PCB_ERR_ARG, "pcb_embed_pos_rows: bad sizes");
+    if (n_rows == 0) return PCB_OK;
+    PCB_REQUIRE(table && ids && out && (!pos_table || (positions && max_positions > 0)), PCB_ERR_ARG, "pcb_embed_pos_rows: null pointer");
+    PCB_REQUIRE(n_streams == 1 || stream_stride >= (int64_t)n_rows * width, PCB_ERR_ARG, "pcb_embed_pos_rows: streams overlap");
+    if (dtype == PCB_BF16)
+        hipLaunchKernelGGL(embed_pos_rows_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)table,
+                           (const bf16_t*)pos_table, ids, positions, out, stream_stride, n_streams, width, vocab, max_positions);
+    else
+        hipLaunchKernelGGL(embed_pos_rows_kernel<float>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, (const float*)table,
+                           (const float*)pos_table, ids, positions, out, stream_stride, n_streams, width, vocab, max_positions);
+    return pcb_check_launch("embed_pos_rows_kernel");
+}
+
+PCB_EXPORT int pcb_hyper_norm(const pcb_hyper_norm_args* a, void* stream) {
+    PCB_REQUIRE(a && a->struct_bytes == sizeof(pcb_hyper_norm_args), PCB_ERR_ARG, "pcb_hyper_norm: struct size mismatch");
+    PCB_REQUIRE(PCB_DTYPE_OK(a->dtype) && a->n_rows >= 0 && a->width > 0 && a->n_streams >= 1 && a->n_streams <= MAX_STREAMS,
+                PCB_ERR_ARG, "pcb_hyper_norm: bad sizes (1 <= streams <= 8)");
+    PCB_REQUIRE(a->norm >= PCB_NORM_NONE && a->norm <= PCB_NORM_DYT, PCB_ERR_ARG, "pcb_hyper_norm: unknown norm");
+    if (a->n_rows == 0) return PCB_OK;
+    PCB_REQUIRE(a->streams && (!a->y || (a->mix && a->out_w)), PCB_ERR_ARG, "pcb_hyper_norm: null pointer");
+    PCB_REQUIRE(!a->out || a->norm == PCB_NORM_NONE || (a->gain && (a->norm != PCB_NORM_DYT || a->alpha)), PCB_ERR_ARG,
+                "pcb_hyper_norm: the norm needs its gain (and alpha)");
+    PCB_REQUIRE(a->norm != PCB_NORM_RMS || a->width <= 16384, PCB_ERR_ARG, "pcb_hyper_norm: width <= 16384 with the RMS norm");
+    const size_t lds = a->norm == PCB_NORM_RMS && a->out ? (size_t)a->width * sizeof(float) : 0;
+    if (a->dtype == PCB_BF16)
+        hipLaunchKernelGGL(hyper_norm_kernel<bf16_t>, dim3(a->n_rows), dim3(256), lds, (hipStream_t)stream, *a);
+    else
+        hipLaunchKernelGGL(hyper_norm_kernel<float>, dim3(a->n_rows), dim3(256), lds, (hipStream_t)stream, *a);
+    return pcb_check_launch("hyper_norm_kernel");
+}
+
+PCB_EXPORT int pcb_gated_norm(const float* x, int64_t ldx, const float* gain, const void* gate, int64_t ldg, void* out, int64_t ldo,
+                              int32_t dtype, float eps, int32_t n_rows, int32_t cols, void* stream) {
+    PCB_REQUIRE(PCB_DTYPE_OK(dtype) && n_rows >= 0 && cols > 0 && ldx >= cols && ldo >= cols && (!gate || ldg >= cols), PCB_ERR_ARG,
+                "pcb_gated_norm: bad sizes");
+    if (n_rows == 0) return PCB_OK;
+    PCB_REQUIRE(x && out, PCB_ERR_ARG, "pcb_gated_norm: null pointer");
+    if (dtype == PCB_BF16)
+        hipLaunchKernelGGL(gated_norm_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const bf16_t*)gate,
+                           ldg, (bf16_t*)out, ldo, eps, cols);
+    else
+        hipLaunchKernelGGL(gated_norm_kernel<float>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, x, ldx, gain, (const float*)gate, ldg,
+                           (float*)out, ldo, eps, cols);
+    return pcb_check_launch("gated_norm_kernel");
+}
+
+PCB_EXPORT int pcb_router_select(const float* logits, int32_t n_rows, int32_t n_out, int32_t top, int32_t score_fn,
+                                 const float* correction, int32_t groups, int32_t groups_keep, int32_t renorm, int32_t* expert,
+                                 float* weight, void* stream) {
+    PCB_REQUIRE(n_rows >= 0 && n_out > 0 && n_out <= 2048 && top > 0 && top <= 64 && top <= n_out, PCB_ERR_ARG,
+                "pcb_router_select: bad sizes (1 <= top <= 64, top <= n_out <= 2048)");
+    PCB_REQUIRE(groups >= 1 && groups <= 64 && n_out % groups == 0 && groups_keep >= 1 && groups_keep <= groups &&
+                    top <= n_out / groups * groups_keep,
+                PCB_ERR_ARG, "pcb_router_select: bad groups (<= 64 equal groups, top within the kept ones)");
+    PCB_REQUIRE(score_fn == PCB_SCORE_SIGMOID || score_fn == PCB_SCORE_SOFTMAX, PCB_ERR_ARG, "pcb_router_select: unknown score function");
+    if (n_rows == 0) return PCB_OK;
+    PCB_REQUIRE(logits && expert && weight, PCB_ERR_ARG, "pcb_router_select: null pointer");
+    hipLaunchKernelGGL(router_select_kernel, dim3(pcb_ceil_div(n_rows, 4)), dim3(256), (size_t)4 * (2 * n_out + 64) * sizeof(float),
+                       (hipStream_t)stream, logits, n_rows, n_out, top, score_fn, correction, groups, groups_keep, renorm, expert, weight);
+    return pcb_check_launch("router_select_kernel");
+}
+
+PCB_EXPORT int pcb_moe_mix(const float* pair_out, const int32_t* expert, const float* weight, const void* h, int32_t dtype, int32_t n_real,
+                           float* y, int32_t n_rows, int32_t width, int32_t top, void* stream) {
+    PCB_REQUIRE(PCB_DTYPE_OK(dtype) && n_rows >= 0 && width > 0 && top > 0 && n_real >= 0, PCB_ERR_ARG, "pcb_moe_mix: bad sizes");
+    if (n_rows == 0) return PCB_OK;
+    PCB_REQUIRE(pair_out && expert && weight && h && y, PCB_ERR_ARG, "pcb_moe_mix: null pointer");
+    if (dtype == PCB_BF16)
+        hipLaunchKernelGGL(moe_mix_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, pair_out, expert, weight,
+                           (const bf16_t*)h, n_real, y, width, top);
+    else
+        hipLaunchKernelGGL(moe_mix_kernel<float>, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, pair_out, expert, weight,
+                           (const float*)h, n_real, y, width, top);
+    return pcb_check_launch("moe_mix_kernel");
+}

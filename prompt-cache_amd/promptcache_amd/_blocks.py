@@ -16,6 +16,10 @@ _lib: Optional[C.CDLL] = None
 
 BF16, F32 = 0, 1
 EPI_STORE, EPI_SILU_MUL, EPI_SCALE_ADD = 0, 1, 2
+ACT_NONE, ACT_SILU, ACT_SIGMOID, ACT_RELU2, ACT_SOFTPLUS, ACT_SOFTCAP = 0, 1, 2, 3, 4, 5
+NORM_NONE, NORM_RMS, NORM_DYT = 0, 1, 2
+SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
+ABI_VERSION = 2
 DTYPES = {torch.bfloat16: BF16, torch.float32: F32}
 
 
@@ -36,7 +40,8 @@ class LinearArgs(C.Structure):
                 ("group_off", _vp), ("n_groups", _i32), ("w_group_stride", _i64),
                 ("y", _vp), ("ldy", _i64), ("out_f32", _i32), ("row_dst", _vp),
                 ("base", _vp), ("ldbase", _i64), ("col_scale", _vp),
-                ("split_n", _i32), ("y2", _vp), ("row_off2", _vp), ("head_dim2", _i32), ("head_stride2", _i64)]
+                ("split_n", _i32), ("y2", _vp), ("row_off2", _vp), ("head_dim2", _i32), ("head_stride2", _i64),
+                ("act", _i32), ("act_split", _i32), ("act2", _i32), ("act_param", _f32)]
 
 
 class AttnTalkArgs(C.Structure):
@@ -48,6 +53,40 @@ class AttnTalkArgs(C.Structure):
                 ("slopes", _vp), ("talk", _vp), ("sink", _i32),
                 ("scratch", _vp), ("scratch_floats", _i64), ("out", _vp), ("ldo", _i64),
                 ("tiles64", _vp), ("n_tiles64", _i32), ("max_tile_rows", _i32)]
+
+
+class HyperNormArgs(C.Structure):
+    """``pcb_hyper_norm_args`` (field for field)."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
+                ("streams", _vp), ("stream_stride", _i64), ("n_streams", _i32),
+                ("y", _vp), ("mix", _vp), ("out_w", _vp), ("in_w", _vp),
+                ("norm", _i32), ("gain", _vp), ("bias", _vp), ("alpha", _vp), ("eps", _f32),
+                ("out", _vp), ("x_out", _vp), ("rows", _vp), ("n_rows", _i32), ("width", _i32)]
+
+
+class AttnSoftmaxArgs(C.Structure):
+    """``pcb_attn_softmax_args`` (field for field)."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
+                ("q", _vp), ("ldq", _i64), ("q_scale", _vp), ("tiles", _vp), ("n_tiles", _i32),
+                ("kcache", _vp), ("vcache", _vp), ("slot_stride", _i64), ("head_stride", _i64), ("row_stride", _i64),
+                ("H", _i32), ("Hkv", _i32), ("dim", _i32), ("vdim", _i32), ("scale", _f32), ("window", _i32),
+                ("gate", _vp), ("ldg", _i64), ("out", _vp), ("ldo", _i64)]
+
+
+class DecayAttnArgs(C.Structure):
+    """``pcb_decay_attn_args`` (field for field)."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
+                ("q", _vp), ("k", _vp), ("v", _vp), ("ldq", _i64), ("ldk", _i64), ("ldv", _i64),
+                ("reqs", _vp), ("n_reqs", _i32), ("state", _vp), ("slot_stride", _i64), ("decay", _vp),
+                ("H", _i32), ("dim", _i32), ("vdim", _i32), ("out", _vp), ("ldo", _i64)]
+
+
+class SelectiveScanArgs(C.Structure):
+    """``pcb_selective_scan_args`` (field for field)."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
+                ("x", _vp), ("ldx", _i64), ("dt", _vp), ("lddt", _i64), ("B", _vp), ("Cm", _vp), ("ldbc", _i64),
+                ("z", _vp), ("ldz", _i64), ("A", _vp), ("D", _vp), ("reqs", _vp), ("n_reqs", _i32),
+                ("state", _vp), ("slot_stride", _i64), ("C", _i32), ("N", _i32), ("out", _vp), ("ldo", _i64)]
 
 
 # name -> (restype, argtypes); mirrors include/promptcache_blocks.h one to one
@@ -63,6 +102,16 @@ SIGNATURES = {
     "pcb_moe_combine": (C.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "pcb_attn_talk_band": (C.c_int32, [_i32, _i32]),
     "pcb_attn_talk": (C.c_int, [C.POINTER(AttnTalkArgs), _vp]),
+    "pcb_embed_pos_rows": (C.c_int, [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "pcb_hyper_norm": (C.c_int, [C.POINTER(HyperNormArgs), _vp]),
+    "pcb_gated_norm": (C.c_int, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32, _f32, _i32, _i32, _vp]),
+    "pcb_router_select": (C.c_int, [_vp, _i32, _i32, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "pcb_moe_mix": (C.c_int, [_vp, _vp, _vp, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _vp]),
+    "pcb_attn_softmax": (C.c_int, [C.POINTER(AttnSoftmaxArgs), _vp]),
+    "pcb_decay_attn": (C.c_int, [C.POINTER(DecayAttnArgs), _vp]),
+    "pcb_causal_conv": (C.c_int, [_vp, _i64, _vp, _vp, _i32, _i32, _vp, _vp, _i64, _vp, _i64, _i32, _i32, _i32, _vp]),
+    "pcb_conv_state_update": (C.c_int, [_vp, _i64, _i32, _vp, _i32, _vp, _i64, _i32, _i32, _vp]),
+    "pcb_selective_scan": (C.c_int, [C.POINTER(SelectiveScanArgs), _vp]),
 }
 
 
@@ -84,7 +133,7 @@ def load(build_missing: bool = True) -> C.CDLL:
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = res, args
-    if lib.pcb_version() != 1:
+    if lib.pcb_version() != ABI_VERSION:
         raise RuntimeError("libpromptcache_blocks.so: ABI version mismatch (rebuild it)")
     _lib = lib
     return lib
@@ -151,8 +200,11 @@ def mix_norm(hist: torch.Tensor, n_streams: int, coef: Optional[torch.Tensor], g
 
 def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, M: int, epilogue: int = EPI_STORE, bias=None, w2=None,
            row_src=None, row_scale=None, group_off=None, n_groups: int = 0, row_dst=None, base=None, col_scale=None,
-           split_n: int = 0, y2=None, row_off2=None, head_dim2: int = 0, head_stride2: int = 0) -> None:
-    """``w``: [N, K], or [groups, N, K] with ``group_off``.  ``x``: [rows, K] of the weights' element type."""
+           split_n: int = 0, y2=None, row_off2=None, head_dim2: int = 0, head_stride2: int = 0, act: int = ACT_NONE,
+           act_split: int = 0, act2: int = ACT_NONE, act_param: float = 0.0, ldy: Optional[int] = None) -> None:
+    """``w``: [N, K], or [groups, N, K] with ``group_off``.  ``x``: [rows, K] of the weights' element type.  ``act`` (and ``act2``
+    from column ``act_split`` on): the element-wise function of a plain store.  ``ldy``: row stride of ``y`` when it is a
+    column block of a wider matrix."""
     code = _code(w)
     assert x.dtype == w.dtype and x.is_contiguous() and w.is_contiguous() and x.is_cuda and w.is_cuda
     N, K = w.shape[-2], w.shape[-1]
@@ -185,13 +237,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, M: int, epilogu
     else:
         assert y.is_contiguous() and (y.dtype == w.dtype or y.dtype == torch.float32)
         cols = split_n if split_n else N
-        assert y.shape[-1] == cols and (row_dst is not None or y.shape[0] >= M)
+        assert (y.shape[-1] == cols or (ldy is not None and ldy >= cols)) and (row_dst is not None or y.shape[0] >= M)
     if split_n:
         _want(row_off2, torch.int64, "linear row_off2")
         assert y2 is not None and y2.dtype == w.dtype and row_off2.numel() >= M and head_dim2 > 0
     a = LinearArgs(C.sizeof(LinearArgs), code, epilogue, _p(x), K, _p(row_src), _p(row_scale), _p(w), _p(w2), K, _p(bias),
-                   M, N, K, _p(group_off), n_groups, N * K if n_groups else 0, _p(y), y.shape[-1], out_f32, _p(row_dst),
-                   _p(base), N, _p(col_scale), split_n, _p(y2), _p(row_off2), head_dim2, head_stride2)
+                   M, N, K, _p(group_off), n_groups, N * K if n_groups else 0, _p(y), y.shape[-1] if ldy is None else ldy, out_f32,
+                   _p(row_dst), _p(base), N, _p(col_scale), split_n, _p(y2), _p(row_off2), head_dim2, head_stride2,
+                   int(act), int(act_split), int(act2), float(act_param))
     check(load().pcb_linear(C.byref(a), _stream()), "pcb_linear")
 
 
@@ -252,3 +305,141 @@ def attn_talk(q: torch.Tensor, tiles: torch.Tensor, n_tiles: int, cache: torch.T
         _want(tiles64, torch.int32, "attn_talk tiles64")
         assert tiles64.numel() >= 4 * n_tiles64 > 0
     check(load().pcb_attn_talk(C.byref(a), _stream()), "pcb_attn_talk")
+
+
+# ---- blocks of designs with several residual streams, gated / recurrent mixers and group-limited routers ----------------------
+def embed_pos_rows(table: torch.Tensor, pos_table: Optional[torch.Tensor], ids: torch.Tensor, positions: Optional[torch.Tensor],
+                   out: torch.Tensor) -> None:
+    """``out`` fp32 [streams, rows, width]: every stream receives table[ids] + pos_table[positions]."""
+    S, n, width = out.shape
+    _want(ids, torch.int32, "embed_pos_rows ids"); _want(out, torch.float32, "embed_pos_rows out")
+    assert ids.numel() >= n and table.shape[1] == width and table.is_contiguous()
+    if pos_table is not None:
+        _want(positions, torch.int32, "embed_pos_rows positions")
+        assert pos_table.dtype == table.dtype and pos_table.shape[1] == width and pos_table.is_contiguous() and positions.numel() >= n
+    check(load().pcb_embed_pos_rows(_p(table), _p(pos_table), _code(table), _p(ids), _p(positions), _p(out), n * width, S, n, width,
+                                    table.shape[0], pos_table.shape[0] if pos_table is not None else 0, _stream()), "pcb_embed_pos_rows")
+
+
+def hyper_norm(streams: torch.Tensor, *, y=None, mix=None, out_w=None, in_w=None, norm: int = NORM_NONE, gain=None, bias=None,
+               alpha=None, eps: float = 1e-6, out=None, x_out=None, rows=None, n_rows: Optional[int] = None) -> None:
+    """``streams`` fp32 [S, T, W].  With ``y`` (fp32 [T, W]) the streams are rewritten through ``mix`` [S, S] / ``out_w`` [S]; with
+    ``out`` (E) or ``x_out`` (fp32) the ``in_w``-weighted sum of the streams is normed and stored (rows ``rows`` only, if given)."""
+    _want(streams, torch.float32, "hyper_norm streams")
+    S, T, W = streams.shape
+    n = (rows.numel() if rows is not None else T) if n_rows is None else n_rows
+    for t, nm in ((y, "y"), (mix, "mix"), (out_w, "out_w"), (in_w, "in_w"), (gain, "gain"), (bias, "bias"), (alpha, "alpha"), (x_out, "x_out")):
+        _want(t, torch.float32, "hyper_norm " + nm)
+    if y is not None:
+        assert y.shape[-1] == W and y.shape[0] >= (T if rows is not None else n) and mix.numel() == S * S and out_w.numel() == S
+    assert in_w is None or in_w.numel() == S
+    assert rows is not None or n <= T
+    if out is not None:
+        assert out.is_contiguous() and out.shape[-1] == W and out.numel() >= n * W
+        if norm != NORM_NONE:
+            assert gain is not None and gain.numel() == W and (bias is None or bias.numel() == W)
+    if x_out is not None:
+        assert x_out.numel() >= n * W
+    if rows is not None:
+        _want(rows, torch.int32, "hyper_norm rows")
+    a = HyperNormArgs(C.sizeof(HyperNormArgs), _code(out) if out is not None else BF16, _p(streams), T * W, S, _p(y), _p(mix), _p(out_w),
+                      _p(in_w), int(norm), _p(gain), _p(bias), _p(alpha), float(eps), _p(out), _p(x_out), _p(rows), n, W)
+    check(load().pcb_hyper_norm(C.byref(a), _stream()), "pcb_hyper_norm")
+
+
+def gated_norm(x: torch.Tensor, gain: Optional[torch.Tensor], gate: Optional[torch.Tensor], ldg: int, out: torch.Tensor, eps: float,
+               n_rows: int) -> None:
+    """``x`` fp32 [rows, cols]; ``gate`` E, a column block (row stride ``ldg``) of a wider matrix; ``out`` E [rows, cols]."""
+    _want(x, torch.float32, "gated_norm x"); _want(gain, torch.float32, "gated_norm gain")
+    cols = x.shape[-1]
+    assert out.is_contiguous() and out.shape[-1] == cols and x.shape[0] >= n_rows and out.shape[0] >= n_rows
+    assert gain is None or gain.numel() == cols
+    if gate is not None:
+        assert gate.dtype == out.dtype and gate.is_cuda and ldg >= cols
+    check(load().pcb_gated_norm(_p(x), cols, _p(gain), _p(gate), ldg, _p(out), cols, _code(out), float(eps), n_rows, cols, _stream()),
+          "pcb_gated_norm")
+
+
+def router_select(logits: torch.Tensor, top: int, expert: torch.Tensor, weight: torch.Tensor, n_rows: int, *, score_fn: int,
+                  correction: Optional[torch.Tensor] = None, groups: int = 1, groups_keep: int = 1, renorm: bool = False) -> None:
+    _want(logits, torch.float32, "router_select logits"); _want(expert, torch.int32, "router_select expert")
+    _want(weight, torch.float32, "router_select weight"); _want(correction, torch.float32, "router_select correction")
+    n_out = logits.shape[-1]
+    assert logits.shape[0] >= n_rows and expert.numel() >= n_rows * top and weight.numel() >= n_rows * top
+    assert correction is None or correction.numel() == n_out
+    check(load().pcb_router_select(_p(logits), n_rows, n_out, top, int(score_fn), _p(correction), groups, groups_keep, int(renorm),
+                                   _p(expert), _p(weight), _stream()), "pcb_router_select")
+
+
+def moe_mix(pair_out: torch.Tensor, expert: torch.Tensor, weight: torch.Tensor, h: torch.Tensor, n_real: int, y: torch.Tensor,
+            n_rows: int, top: int) -> None:
+    _want(pair_out, torch.float32, "moe_mix pair_out"); _want(expert, torch.int32, "moe_mix expert")
+    _want(weight, torch.float32, "moe_mix weight"); _want(y, torch.float32, "moe_mix y")
+    W = y.shape[-1]
+    assert pair_out.shape[-1] == W and pair_out.shape[0] >= n_rows * top and h.shape[-1] == W and h.shape[0] >= n_rows and h.is_contiguous()
+    assert y.shape[0] >= n_rows and expert.numel() >= n_rows * top and weight.numel() >= n_rows * top
+    check(load().pcb_moe_mix(_p(pair_out), _p(expert), _p(weight), _p(h), _code(h), n_real, _p(y), n_rows, W, top, _stream()), "pcb_moe_mix")
+
+
+def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, kcache: torch.Tensor, v_offset: int, slot_stride: int,
+                 head_stride: int, row_stride: int, H: int, Hkv: int, dim: int, vdim: int, scale: float, out: torch.Tensor, *,
+                 q_scale: Optional[torch.Tensor] = None, window: int = 0, gate: Optional[torch.Tensor] = None, ldg: int = 0) -> None:
+    """``q``: E rows (row stride ``ldq``, head h at column h * dim); ``kcache``: the plane that holds the keys, the values
+    ``v_offset`` elements behind them; ``gate``: E rows of stride ``ldg``; ``out`` E [rows, H * vdim]."""
+    _want(tiles, torch.int32, "attn_softmax tiles"); _want(q_scale, torch.float32, "attn_softmax q_scale")
+    assert q.dtype == kcache.dtype == out.dtype and out.is_contiguous() and kcache.is_cuda and q.is_cuda
+    assert tiles.numel() >= 4 * n_tiles and out.shape[-1] == H * vdim and ldq >= H * dim
+    assert gate is None or (gate.dtype == q.dtype and ldg >= H * vdim)
+    es = kcache.element_size()
+    a = AttnSoftmaxArgs(C.sizeof(AttnSoftmaxArgs), _code(q), _p(q), ldq, _p(q_scale), _p(tiles), n_tiles, _p(kcache),
+                        kcache.data_ptr() + v_offset * es, slot_stride, head_stride, row_stride, H, Hkv, dim, vdim, float(scale),
+                        int(window), _p(gate), ldg, _p(out), out.shape[-1])
+    check(load().pcb_attn_softmax(C.byref(a), _stream()), "pcb_attn_softmax")
+
+
+def decay_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ld: int, reqs: torch.Tensor, n_reqs: int, state: torch.Tensor,
+               decay: torch.Tensor, H: int, dim: int, vdim: int, out: torch.Tensor) -> None:
+    """``q``, ``k``, ``v``: column blocks (row stride ``ld``) of one E matrix; ``state`` fp32 [slots, H, dim, vdim]; ``out`` fp32
+    [rows, H * vdim]."""
+    _want(reqs, torch.int32, "decay_attn reqs"); _want(state, torch.float32, "decay_attn state"); _want(decay, torch.float32, "decay_attn decay")
+    _want(out, torch.float32, "decay_attn out")
+    assert q.dtype == k.dtype == v.dtype and q.is_cuda and reqs.numel() >= 4 * n_reqs and decay.numel() == H
+    assert tuple(state.shape[1:]) == (H, dim, vdim) and out.shape[-1] == H * vdim
+    a = DecayAttnArgs(C.sizeof(DecayAttnArgs), _code(q), _p(q), _p(k), _p(v), ld, ld, ld, _p(reqs), n_reqs, _p(state), H * dim * vdim,
+                      _p(decay), H, dim, vdim, _p(out), out.shape[-1])
+    check(load().pcb_decay_attn(C.byref(a), _stream()), "pcb_decay_attn")
+
+
+def causal_conv(x: torch.Tensor, ldx: int, w: torch.Tensor, bias: Optional[torch.Tensor], silu: bool, row_meta: torch.Tensor,
+                state: torch.Tensor, out: torch.Tensor, n_rows: int) -> None:
+    """``x``: E rows (stride ``ldx``) of C channels; ``w`` E [C, taps]; ``state`` E [slots, taps - 1, C]; ``out`` E [rows, C]."""
+    C_, taps = w.shape
+    _want(row_meta, torch.int32, "causal_conv row_meta")
+    assert x.dtype == w.dtype == out.dtype == state.dtype and out.is_contiguous() and out.shape[-1] == C_ and w.is_contiguous()
+    assert row_meta.numel() >= 4 * n_rows and tuple(state.shape[1:]) == (taps - 1, C_) and (bias is None or bias.numel() == C_)
+    check(load().pcb_causal_conv(_p(x), ldx, _p(w), _p(bias), _code(x), int(silu), _p(row_meta), _p(state), (taps - 1) * C_, _p(out),
+                                 C_, n_rows, C_, taps, _stream()), "pcb_causal_conv")
+
+
+def conv_state_update(x: torch.Tensor, ldx: int, reqs: torch.Tensor, n_reqs: int, state: torch.Tensor) -> None:
+    _want(reqs, torch.int32, "conv_state_update reqs")
+    taps, C_ = state.shape[1] + 1, state.shape[2]
+    assert x.dtype == state.dtype and reqs.numel() >= 4 * n_reqs and state.is_contiguous()
+    check(load().pcb_conv_state_update(_p(x), ldx, _code(x), _p(reqs), n_reqs, _p(state), (taps - 1) * C_, C_, taps, _stream()),
+          "pcb_conv_state_update")
+
+
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, z: Optional[torch.Tensor], ldz: int, A: torch.Tensor,
+                   D: Optional[torch.Tensor], reqs: torch.Tensor, n_reqs: int, state: torch.Tensor, out: torch.Tensor) -> None:
+    """``x`` E [rows, C]; ``dt`` fp32 [rows, C]; ``bc`` fp32 [rows, 2 N] = B | C; ``z`` E rows of stride ``ldz``; ``A`` fp32 [C, N];
+    ``state`` fp32 [slots, C, N]; ``out`` E [rows, C]."""
+    C_, N = A.shape
+    for t, nm in ((dt, "dt"), (bc, "bc"), (A, "A"), (D, "D"), (state, "state")):
+        _want(t, torch.float32, "selective_scan " + nm)
+    _want(reqs, torch.int32, "selective_scan reqs")
+    assert x.dtype == out.dtype and x.is_contiguous() and out.is_contiguous() and x.shape[-1] == C_ == out.shape[-1] == dt.shape[-1]
+    assert bc.shape[-1] == 2 * N and tuple(state.shape[1:]) == (C_, N) and reqs.numel() >= 4 * n_reqs
+    assert z is None or (z.dtype == x.dtype and ldz >= C_)
+    a = SelectiveScanArgs(C.sizeof(SelectiveScanArgs), _code(x), _p(x), C_, _p(dt), C_, _p(bc), bc.data_ptr() + 4 * N, 2 * N, _p(z), ldz,
+                          _p(A), _p(D), _p(reqs), n_reqs, _p(state), C_ * N, C_, N, _p(out), C_)
+    check(load().pcb_selective_scan(C.byref(a), _stream()), "pcb_selective_scan")

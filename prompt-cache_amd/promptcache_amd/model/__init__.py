@@ -22,7 +22,7 @@ from typing import Callable, List, Optional, Tuple
 import torch
 
 from ..pml import Preprocessor, PreprocessorList, escape_xml  # noqa: F401  (re-exported like the reference)
-from .config import FALCON_SHAPES, MPT_SHAPES, SHAPES, FalconShape, KazolornShape, LlamaShape, MptShape, architecture_of
+from .config import FALCON_SHAPES, MPT_SHAPES, SHAPES, DibizenShape, FalconShape, KazolornShape, LlamaShape, MptShape, architecture_of
 from .tokenizer import StandInTokenizer
 
 # HF hub ids the reference's drivers use (demo.py:27, eval.py:36, config/*.json) -> shape presets
@@ -321,7 +321,47 @@ class Kazolorn(LanguageModel):
         return [t % self.config.vocab_size for t in super().encode(text)]
 
 
-ADAPTERS = {"llama": Llama2, "falcon": Falcon, "mpt": Mpt, "kazolorn": Kazolorn}
+class Dibizen(LanguageModel):
+    """Adapter of the Dibizen design (``config.DibizenShape``, ``dibizen_hip.DibizenHIP``).  A checkpoint directory holds
+    ``config.json`` and ``model.safetensors``; without one, ``shape=`` plus ``random_init=True`` (or ``weights=``) gives seeded
+    random weights.  ``dtype``: ``torch.bfloat16`` (serving) or ``torch.float32`` (everything in true 32-bit)."""
+
+    def __init__(self, name: Optional[str] = None, device: str = "cuda:0", shape: Optional[DibizenShape] = None,
+                 weights=None, tokenizer=None, random_init: bool = False, seed: int = 0, dtype=torch.bfloat16, **_kwargs):
+        from .dibizen_hip import DibizenHIP
+        from . import weights as W
+
+        if weights is not None:
+            assert shape is not None, "pass shape= together with weights="
+        elif name is not None and os.path.isdir(name):
+            shape = shape or DibizenShape.from_dir(name)
+            weights = W.load_dibizen_safetensors(name, shape)
+        else:
+            if shape is None or not random_init:
+                raise FileNotFoundError(f"no checkpoint directory {name!r}: pass one, or shape= with random_init=True")
+            weights = W.make_dibizen_weights(shape, seed, device=device)
+        if tokenizer is None:
+            tokenizer = StandInTokenizer(max(shape.vocab_size, 512))
+        model = DibizenHIP(shape, weights, device=device, dtype=dtype)
+        self.formatter = FormatConversation(system=("", "\n\n", ""), user=("User: ", "\n\nAssistant:"), assistant=(" ", "\n\n"))
+        super().__init__(name or shape.name, model, tokenizer, [tokenizer.eos_token_id], [])
+
+    def get_formatter(self) -> Callable[[str], str]:
+        return self.formatter
+
+    def get_cache_shape(self) -> Tuple[int, int, int]:
+        """(layers, kv heads, key size) of the first attention layer that keeps a cache (zeros when no layer does); the other
+        layers keep states of their own shapes (``DibizenHIP.new_arena`` knows them all)."""
+        for l in self.config.layers:
+            if l.kind == "attention" and l.kv_from < 0:
+                return len(self.config.layers), l.kv_heads, l.dim
+        return len(self.config.layers), 0, 0
+
+    def encode(self, text: str) -> List[int]:
+        return [t % self.config.vocab_size for t in super().encode(text)]
+
+
+ADAPTERS = {"llama": Llama2, "falcon": Falcon, "mpt": Mpt, "kazolorn": Kazolorn, "dibizen": Dibizen}
 
 
 def load_language_model(path: str, **kwargs) -> LanguageModel:

@@ -31,7 +31,7 @@ import torch
 from .. import _blocks as B
 from .config import KazolornShape
 from .kv_arena import SlotArena
-from .llama_hip import CausalLMOutput
+from .slot_model import SlotKV, SlotModel  # noqa: F401  (SlotKV is re-exported)
 
 ATTN_SCRATCH_FLOATS = 1 << 28          # the score band of one attention call is kept below 1 GiB (more rows: several calls)
 
@@ -41,25 +41,7 @@ def distance_slopes(heads: int) -> torch.Tensor:
     return torch.tensor([2.0 ** (-8.0 * (h + 1) / heads) for h in range(heads)], dtype=torch.float32)
 
 
-class SlotKV:
-    """``past_key_values`` of this model: the arena and the slots of the batch rows, in order."""
-
-    def __init__(self, arena: SlotArena, slots: List[int]):
-        self.arena, self.slots = arena, list(slots)
-
-    def __len__(self):
-        return len(self.arena.planes)
-
-    def __del__(self):
-        try:
-            for s in self.slots:
-                if s in self.arena._live:
-                    self.arena.free(s)
-        except Exception:
-            pass
-
-
-class KazolornHIP:
+class KazolornHIP(SlotModel):
     def __init__(self, shape: KazolornShape, weights: Dict[str, torch.Tensor], device="cuda:0", dtype=torch.bfloat16,
                  decode_headroom: int = 256):
         if dtype not in (torch.bfloat16, torch.float32):
@@ -117,19 +99,6 @@ class KazolornHIP:
 
     def kv_bytes_per_token(self) -> int:
         return sum(l.kv_heads * l.dim for l in self.config.layers) * (2 if self.dtype == torch.bfloat16 else 4)
-
-    # ---- scratch -----------------------------------------------------------------------------------------------------------
-    def _scratch(self, name: str, numel: int, dtype) -> torch.Tensor:
-        """A named scratch buffer of at least ``numel`` elements (grown by doubling, never shrunk)."""
-        t = self._buf.get(name)
-        if t is None or t.numel() < numel or t.dtype != dtype:
-            n = max(numel, 2 * t.numel() if t is not None and t.dtype == dtype else 0, 1024)
-            t = torch.empty(n, dtype=dtype, device=self.device)
-            self._buf[name] = t
-        return t
-
-    def _mat(self, name: str, rows: int, cols: int, dtype) -> torch.Tensor:
-        return self._scratch(name, max(rows, 1) * cols, dtype)[:max(rows, 1) * cols].view(max(rows, 1), cols)
 
     # ---- one step ------------------------------------------------------------------------------------------------------------
     @torch.inference_mode()
@@ -339,43 +308,3 @@ class KazolornHIP:
             part_d = torch.from_numpy(part.reshape(-1)).to(self.device)
             B.attn_talk(q[r0:], part_d, part.shape[0], plane, arena.slot_stride(i), arena.head_stride(i), l.heads, l.kv_heads, l.dim,
                         l.scale, l.window, max_kv, lw["slopes"], lw["talk"], True, scratch, att[r0:])
-
-    # ---- the adapters' calling convention --------------------------------------------------------------------------------------
-    @torch.inference_mode()
-    def __call__(self, input_ids: torch.Tensor, position_ids: Optional[torch.Tensor] = None, past_key_values=None,
-                 attention_mask: Optional[torch.Tensor] = None, use_cache: bool = True, last_token_only: bool = False,
-                 num_layers: Optional[int] = None, **_unused) -> CausalLMOutput:
-        """``input_ids`` [B, q]; right padding is described by ``attention_mask`` [B, q] (1 = token).  Positions count from 0 in
-        each sequence and enter only as distances, so ``position_ids`` are not needed (they are accepted and ignored).
-        Logits come back as [B, q, vocab] (padded places hold zeros), or [B, 1, vocab] with ``last_token_only``."""
-        ids = input_ids.detach().to("cpu").reshape(input_ids.shape[0], -1)
-        Bn, q_len = ids.shape
-        if attention_mask is not None:
-            am = attention_mask.detach().to("cpu").reshape(Bn, -1)[:, -q_len:]
-            if bool((am[:, 1:] > am[:, :-1]).any()):
-                raise NotImplementedError("left / interior padding masks are not supported")
-            counts = [int(c) for c in am.sum(dim=1)]
-        else:
-            counts = [q_len] * Bn
-        if past_key_values is None:
-            arena = self.default_arena
-            if arena is None:
-                arena = self.default_arena = self.new_arena(Bn, q_len + self.decode_headroom)
-            past_key_values = SlotKV(arena, [arena.alloc() for _ in range(Bn)])
-        elif not isinstance(past_key_values, SlotKV) or len(past_key_values.slots) != Bn:
-            raise ValueError("past_key_values must be what an earlier call of this model returned, for the same batch")
-        arena, slots = past_key_values.arena, past_key_values.slots
-        toks = [ids[b, :counts[b]].tolist() for b in range(Bn)]
-        want = [[c - 1] for c in counts] if last_token_only else [list(range(c)) for c in counts]
-        flat = self.forward_rows(arena, slots, toks, want, num_layers=num_layers)
-        if last_token_only:
-            logits = flat.view(Bn, 1, self.V)
-        elif all(c == q_len for c in counts):
-            logits = flat.view(Bn, q_len, self.V)
-        else:
-            logits = torch.zeros((Bn, q_len, self.V), dtype=torch.float32, device=self.device)
-            at = 0
-            for b, c in enumerate(counts):
-                logits[b, :c] = flat[at:at + c]
-                at += c
-        return CausalLMOutput(logits=logits, past_key_values=past_key_values if use_cache else None)

@@ -286,10 +286,17 @@ class SlotArena:
     back (``free``); a freed slot is handed out again with length 0, its old rows are simply overwritten.
 
     Rows are addressed by position (row j of a slot holds position j): nothing in the layout depends on how a sequence was cut
-    into steps or on which slot it sits in.  ``reserve`` grows the planes (more slots, longer rows) keeping every live row."""
+    into steps or on which slot it sits in.  ``reserve`` grows the planes (more slots, longer rows) keeping every live row.
 
-    def __init__(self, layer_dims, slots: int, cap: int, device, dtype=torch.bfloat16):
+    A layer may also (or instead: ``(0, 0)`` key dims) carry STATES of a fixed size per slot -- a recurrent mixer's matrix, the
+    last inputs of a short convolution: ``states[layer]`` lists ``(shape, dtype)`` pairs, kept as tensors ``[slots, *shape]`` in
+    ``self.states[layer]``.  A state is not cleared when its slot changes hands: whoever reads it treats a request that starts
+    at position 0 as starting from zero."""
+
+    def __init__(self, layer_dims, slots: int, cap: int, device, dtype=torch.bfloat16, states=None):
         self.layer_dims = [(int(g), int(d)) for g, d in layer_dims]
+        self.state_specs = [[(tuple(int(v) for v in shp), dt) for shp, dt in (per or [])] for per in (states or [[]] * len(self.layer_dims))]
+        self.states: List[List[torch.Tensor]] = [[] for _ in self.state_specs]
         self.device, self.dtype = torch.device(device), dtype
         self.slots, self.cap = 0, 0
         self.planes: List[torch.Tensor] = []
@@ -310,6 +317,16 @@ class SlotArena:
     def bytes_per_token(self) -> int:
         return sum(g * d for g, d in self.layer_dims) * torch.empty(0, dtype=self.dtype).element_size()
 
+    def state_bytes_per_slot(self) -> int:
+        n = 0
+        for per in self.state_specs:
+            for shp, dt in per:
+                k = 1
+                for v in shp:
+                    k *= v
+                n += k * torch.empty(0, dtype=dt).element_size()
+        return n
+
     def reserve(self, slots: int, cap: int) -> None:
         """At least ``slots`` slots of at least ``cap`` positions each."""
         slots, cap = max(slots, self.slots), max(cap, self.cap)
@@ -320,6 +337,12 @@ class SlotArena:
         if keep:
             for old, nw in zip(self.planes, new):
                 nw[:self.slots, :, :keep].copy_(old[:, :, :keep])
+        if slots != self.slots:
+            grown = [[torch.zeros((slots, *shp), device=self.device, dtype=dt) for shp, dt in per] for per in self.state_specs]
+            for old_l, new_l in zip(self.states, grown):
+                for old, nw in zip(old_l, new_l):
+                    nw[:self.slots].copy_(old)
+            self.states = grown
         self._free += list(range(self.slots, slots))
         self.lengths += [0] * (slots - self.slots)
         self.planes, self.slots, self.cap = new, slots, cap

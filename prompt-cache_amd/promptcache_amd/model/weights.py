@@ -328,3 +328,112 @@ def load_kazolorn_safetensors(path: str, cfg):
         if tuple(raw[k].shape) != tuple(shp):
             raise ValueError(f"{path}: {k} has shape {tuple(raw[k].shape)}, the configuration implies {tuple(shp)}")
     return {k: raw[k] for k in want}
+
+
+def dibizen_weight_shapes(cfg) -> Dict[str, tuple]:
+    """Tensor names and shapes of a Dibizen checkpoint (``model.safetensors``): ``embed``, ``pos``; per layer ``l{i}.norm1|norm2``
+    (each with ``.b`` and a scalar ``.alpha``), ``l{i}.hc1|hc2.in|out|mix`` (hyper-connection weights of the two sublayers), the
+    mixer's ``l{i}.mix.*`` (lightning: ``q k v g o norm``; attention: ``q g o`` and, unless it borrows another layer's cache,
+    ``k v``; mamba1: ``in conv conv.b x dt dt.b A_log D o``) and the feed-forward's ``l{i}.mlp.router|correction`` and
+    ``l{i}.mlp.e{j}.up|down``; then ``final.norm`` (``.b``, ``.alpha``) and ``head``."""
+    W, S = cfg.hidden_size, cfg.streams
+    s = {"embed": (cfg.vocab_size, W), "pos": (cfg.max_positions, W)}
+
+    def norm(name):
+        s[name], s[name + ".b"], s[name + ".alpha"] = (W,), (W,), ()
+
+    def hyper(name):
+        s[name + ".in"], s[name + ".out"], s[name + ".mix"] = (S,), (S,), (S, S)
+
+    for i, l in enumerate(cfg.layers):
+        p = f"l{i}."
+        norm(p + "norm1")
+        hyper(p + "hc1")
+        m = p + "mix."
+        if l.kind == "lightning":
+            s[m + "q"], s[m + "k"] = (l.heads * l.dim, W), (l.heads * l.dim, W)
+            s[m + "v"], s[m + "g"] = (l.heads * l.vdim, W), (l.heads * l.vdim, W)
+            s[m + "o"], s[m + "norm"] = (W, l.heads * l.vdim), (l.heads * l.vdim,)
+        elif l.kind == "attention":
+            s[m + "q"], s[m + "g"], s[m + "o"] = (l.heads * l.dim, W), (l.heads * l.vdim, W), (W, l.heads * l.vdim)
+            if l.kv_from < 0:
+                s[m + "k"], s[m + "v"] = (l.kv_heads * l.dim, W), (l.kv_heads * l.vdim, W)
+        else:
+            s[m + "in"], s[m + "conv"], s[m + "conv.b"] = (2 * l.inner, W), (l.inner, l.conv), (l.inner,)
+            s[m + "x"], s[m + "dt"], s[m + "dt.b"] = (l.dt_rank + 2 * l.state, l.inner), (l.inner, l.dt_rank), (l.inner,)
+            s[m + "A_log"], s[m + "D"], s[m + "o"] = (l.inner, l.state), (l.inner,), (W, l.inner)
+        if l.experts + l.identity:
+            norm(p + "norm2")
+            hyper(p + "hc2")
+            s[p + "mlp.router"], s[p + "mlp.correction"] = (l.experts + l.identity, W), (l.experts + l.identity,)
+            for e in range(l.experts):
+                s[p + f"mlp.e{e}.up"], s[p + f"mlp.e{e}.down"] = (l.ff, W), (W, l.ff)
+    norm("final.norm")
+    s["head"] = (cfg.vocab_size, W)
+    return s
+
+
+def make_dibizen_weights(cfg, seed: int = 0, device="cpu", scale: float = 1.0):
+    """Seeded random weights (bfloat16 torch tensors) with nothing at a value that would hide a dropped term: norm gains around
+    1 with non-zero biases and an alpha that keeps tanh off its flat part, stream weights that differ between streams, router
+    corrections large enough to change choices, A_log / dt biases that give decays between 0 and 1."""
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    on_gpu = str(device) != "cpu"
+    gd = torch.Generator(device=device).manual_seed(seed) if on_gpu else g
+
+    def rnd(shape, big=False):
+        if big and on_gpu:
+            return torch.randn(shape, generator=gd, device=device, dtype=torch.float32)
+        return torch.randn(shape, generator=g, dtype=torch.float32).to(device)
+
+    out = {}
+    S = cfg.streams
+    for name, shp in dibizen_weight_shapes(cfg).items():
+        leaf = name.split(".", 1)[-1] if name.startswith("l") and name[1].isdigit() else name
+        if leaf.endswith(".alpha"):
+            w = torch.tensor(0.6, device=device) + 0.1 * rnd(shp)
+        elif leaf in ("norm1", "norm2", "final.norm", "mix.norm"):
+            w = 1.0 + 0.1 * rnd(shp)
+        elif leaf in ("hc1.in", "hc2.in"):
+            w = 1.0 / S + 0.2 * rnd(shp)
+        elif leaf in ("hc1.out", "hc2.out"):
+            w = 1.0 + 0.3 * rnd(shp)
+        elif leaf in ("hc1.mix", "hc2.mix"):
+            w = torch.eye(S, device=device) + 0.15 * rnd(shp)
+        elif leaf == "mlp.correction":
+            w = 0.05 * rnd(shp)
+        elif leaf == "mix.A_log":
+            w = torch.log(torch.arange(1, shp[1] + 1, dtype=torch.float32, device=device)).expand(shp) + 0.1 * rnd(shp)
+        elif leaf == "mix.dt.b":
+            w = -2.0 + 0.5 * rnd(shp)
+        elif leaf == "mix.D":
+            w = 1.0 + 0.2 * rnd(shp)
+        elif leaf == "mix.conv":
+            w = 0.5 * rnd(shp)
+        elif leaf.endswith(".b"):
+            w = 0.1 * rnd(shp)
+        elif leaf == "embed":
+            w = rnd(shp, big=True)
+        elif leaf == "pos":
+            w = 0.5 * rnd(shp, big=True)
+        else:
+            w = (scale / (shp[-1] ** 0.5)) * rnd(shp, big=True)
+        out[name] = w.to(torch.bfloat16)
+    return out
+
+
+def load_dibizen_safetensors(path: str, cfg):
+    """The tensors of ``<path>/model.safetensors`` by their own names, on the host, checked against the shapes the
+    configuration implies."""
+    raw = read_checkpoint_dir(path)
+    want = dibizen_weight_shapes(cfg)
+    missing = [k for k in want if k not in raw]
+    if missing:
+        raise KeyError(f"{path}: tensors missing for this configuration: {missing[:6]}{' ...' if len(missing) > 6 else ''}")
+    for k, shp in want.items():
+        if k == "pos" and raw[k].dim() == 2 and raw[k].shape[1] == shp[1]:
+            continue                                  # (the table's own length says how many positions there are)
+        if tuple(raw[k].shape) != tuple(shp):
+            raise ValueError(f"{path}: {k} has shape {tuple(raw[k].shape)}, the configuration implies {tuple(shp)}")
+    return {k: raw[k] for k in want}
