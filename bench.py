@@ -672,6 +672,79 @@ def plan_only(args):
     print(json.dumps(out))
 
 
+def slot_model_case(lm, V, T, steps, warm, g):
+    """Prefill (one prompt of T tokens) and decode (1 and 8 requests at a context of T) throughput of a flat-row model."""
+    import torch
+    m = lm.hf_model
+    prompt = torch.randint(0, V, (T,), generator=g).tolist()
+    res = {}
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    def prefill():
+        ar = m.new_arena(1, T)
+        m.forward_rows(ar, [ar.alloc()], [prompt])
+    for _ in range(warm):
+        prefill()
+    res["prefill_tok_s"] = round(T / timed(prefill, steps), 1)
+    for nb in (1, 8):
+        ar = m.new_arena(nb, T + 4 * (steps + warm) + 8)
+        slots = [ar.alloc() for _ in range(nb)]
+        m.forward_rows(ar, slots, [prompt] * nb)
+        step = lambda: m.forward_rows(ar, slots, [[7]] * nb)
+        for _ in range(warm):
+            step()
+        res[f"decode_b{nb}_tok_s"] = round(nb / timed(step, steps), 1)
+    del lm, m
+    torch.cuda.empty_cache()
+    return res
+
+
+def run_dibizen(args):
+    """Throughput of the Dibizen stack beside the Kazolorn stack (the closest existing model: the same building-block library,
+    bf16 tensors, an fp32 residual, sparse feed-forwards) at equal width, heads, depth and experts.
+
+    Per size: one prompt of 2048 tokens (tokens/s of the prefill), then decoding at a context of 2048 with 1 and 8 requests.
+    `mixed` = lightning, attention, mamba1, attention (borrowing the first one's keys and values); `attention` / `lightning` /
+    `mamba1` = four layers of that mixer alone, which is what prices each mixer's kernels.  Random weights, synthetic tokens."""
+    import torch
+    import __graft_entry__ as ge
+    ge.build()
+    from promptcache_amd.model import Dibizen, Kazolorn
+    from promptcache_amd.model.config import DibizenShape, KazolornShape
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    sizes = {"2k": dict(width=2048, heads=16, kv=4, experts=16, top=2, eff=2048),
+             "4k": dict(width=4096, heads=32, kv=8, experts=16, top=2, eff=4096)}
+    L, V, T, steps, warm = 4, 32000, 2048, max(4, min(args.steps, 20)), max(1, min(args.warmup, 3))
+    g = torch.Generator().manual_seed(0)
+    out = {"metric": "dibizen_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "layers": L, "prompt": T, "sizes": {}}
+    patterns = {"mixed": ["lightning", "attention", "mamba1", "attention"], "attention": ["attention"] * L, "lightning": ["lightning"] * L,
+                "mamba1": ["mamba1"] * L}
+    for key in args.dibizen_sizes.split(","):
+        c = sizes[key]
+        w, h = c["width"], c["heads"]
+        kz = KazolornShape.uniform(V, w, L, h, c["kv"], w // h, 0, 4 * w, experts=c["experts"], top=c["top"], expert_ff=c["eff"],
+                                   dense_first=0, name=f"kazolorn-{key}")
+        row = {"width": w, "heads": h,
+               "kazolorn": slot_model_case(Kazolorn(shape=kz, random_init=True, seed=0, device=dev), V, T, steps, warm, g)}
+        for pk in args.dibizen_patterns.split(","):
+            shape = DibizenShape.uniform(V, w, patterns[pk], h, c["kv"], w // h, c["experts"], c["top"], c["eff"], identity=2, groups=3,
+                                         groups_keep=2, streams=2, inner=2 * w, state=16, max_positions=T + 256, name=f"dibizen-{key}-{pk}")
+            if pk == "mixed":
+                shape.layers[3].kv_from, shape.layers[3].qt_coef, shape.layers[3].qt_every = 1, shape.layers[1].qt_coef, shape.layers[1].qt_every
+            row["dibizen_" + pk] = slot_model_case(Dibizen(shape=shape, random_init=True, seed=0, device=dev), V, T, steps, warm, g)
+        out["sizes"][key] = row
+        print(json.dumps({key: row}), file=sys.stderr, flush=True)
+    print(json.dumps(out))
+
+
 def run_kazolorn(args):
     """Throughput of the Kazolorn stack beside the MPT stack at equal width, heads, depth and feed-forward width.
 
@@ -701,28 +774,7 @@ def run_kazolorn(args):
         return (time.perf_counter() - t0) / n
 
     def kz_case(shape):
-        lm = Kazolorn(shape=shape, random_init=True, seed=0, device=dev)
-        m = lm.hf_model
-        prompt = torch.randint(0, V, (T,), generator=g).tolist()
-        res = {}
-
-        def prefill():
-            ar = m.new_arena(1, T)
-            m.forward_rows(ar, [ar.alloc()], [prompt])
-        for _ in range(warm):
-            prefill()
-        res["prefill_tok_s"] = round(T / timed(prefill, steps), 1)
-        for nb in (1, 8):
-            ar = m.new_arena(nb, T + 4 * (steps + warm) + 8)
-            slots = [ar.alloc() for _ in range(nb)]
-            m.forward_rows(ar, slots, [prompt] * nb)
-            step = lambda: m.forward_rows(ar, slots, [[7]] * nb)
-            for _ in range(warm):
-                step()
-            res[f"decode_b{nb}_tok_s"] = round(nb / timed(step, steps), 1)
-        del lm, m
-        torch.cuda.empty_cache()
-        return res
+        return slot_model_case(Kazolorn(shape=shape, random_init=True, seed=0, device=dev), V, T, steps, warm, g)
 
     def mpt_case(width, heads):
         shape = MptShape(vocab_size=V, hidden_size=width, num_hidden_layers=L, num_attention_heads=heads, name="mpt-eq")
@@ -791,12 +843,20 @@ def main():
                     help="instead of the default workload: prefill / decode throughput of the Kazolorn design at layer sizes of "
                          "real models (random weights), beside the MPT stack (the closest existing model) at equal size")
     ap.add_argument("--kazolorn-sizes", default="2k,4k", help="--kazolorn: which sizes (2k, 4k)")
+    ap.add_argument("--dibizen", action="store_true",
+                    help="instead of the default workload: prefill / decode throughput of the Dibizen design at layer sizes of "
+                         "real models (random weights), beside the Kazolorn stack (the closest existing model) at equal size")
+    ap.add_argument("--dibizen-sizes", default="2k,4k", help="--dibizen: which sizes (2k, 4k)")
+    ap.add_argument("--dibizen-patterns", default="mixed,attention,lightning,mamba1", help="--dibizen: which layer patterns")
     args = ap.parse_args()
     if args.plan_only:
         plan_only(args)
         return
     if args.kazolorn:
         run_kazolorn(args)
+        return
+    if args.dibizen:
+        run_dibizen(args)
         return
 
     import torch

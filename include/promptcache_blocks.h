@@ -255,6 +255,10 @@ typedef struct pcb_attn_softmax_args {
     int64_t ldg;
     void* out;
     int64_t ldo;
+    int32_t n_splits; /* > 1: every (tile, head) is cut into n_splits runs of key blocks that run as workgroups of their own and
+                         leave (maximum, denominator, weighted values) in `part`; a second launch merges them.  For steps of few
+                         rows over long caches. */
+    float* part;      /* fp32 [rows][H][n_splits][vdim + 2], rows = the flat rows the tiles cover (row index = flat row) */
 } pcb_attn_softmax_args;
 int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream);
 
@@ -263,7 +267,8 @@ int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream);
  * q, k: E rows with head h at column h * dim; v: head h at column h * vdim; out fp32 [rows][ldo].  request r = {slot, first
  * position, tokens, first flat row} (int32 x 4, device): its tokens are consecutive rows; a request that starts at position 0
  * starts from a zero state whatever the slot held.  state: fp32 [slots][H][dim][vdim] (slot_stride floats per slot), read at the
- * start and written at the end of each request.  All products run on the fp32 matrix cores.  dim <= 256. */
+ * start and written at the end of each request.  All products run on the fp32 matrix cores.  dim <= 256.
+ * out null: only the states move (the first pass of a segmented prefill, see pcb_state_chain). */
 typedef struct pcb_decay_attn_args {
     uint32_t struct_bytes;
     int32_t dtype;
@@ -297,7 +302,8 @@ int pcb_conv_state_update(const void* x, int64_t ldx, int32_t dtype, const int32
  *   S[c][n] <- exp(dt[c] * A[c][n]) * S[c][n] + dt[c] * x[c] * B[n],   y[c] = sum_n S[c][n] * Cm[n] + D[c] * x[c],
  *   out[c] = y[c] * silu(z[c])   (z null: out = y)
  * per token, in order, for each request {slot, first position, tokens, first flat row}.  x, z: E rows; dt, B, Cm: fp32 rows;
- * A fp32 [C][N], D fp32 [C]; state fp32 [slots][C][N] (zero before position 0); out E.  N <= 256. */
+ * A fp32 [C][N], D fp32 [C]; state fp32 [slots][C][N] (zero before position 0); out E.  N <= 256.
+ * out null: only the states move; dt_sum (fp32 [n_reqs][C], optional) receives each request's sum of dt per channel. */
 typedef struct pcb_selective_scan_args {
     uint32_t struct_bytes;
     int32_t dtype;
@@ -319,8 +325,20 @@ typedef struct pcb_selective_scan_args {
     int32_t C, N;
     void* out;
     int64_t ldo;
+    float* dt_sum;
 } pcb_selective_scan_args;
 int pcb_selective_scan(const pcb_selective_scan_args* a, void* stream);
+
+/* Segmented prefill of a linear recurrence S <- f S + (input term), f = exp(coef * x): a long sequence is cut into segments, a
+ * first pass runs every segment from a ZERO state (local[g] = its own contribution), this call chains them, and a second pass runs
+ * every segment from its true start state.  For chain c = {slot, first position, first segment, segments} (int32 x 4), element-wise
+ * over `elems` floats e:
+ *   s = first position > 0 ? state[slot][e] : 0
+ *   for g = first segment ..:   start[g][e] = s;   s = exp(coef[e] * x[g][e / group]) * s + local[g][e]
+ *   state[slot][e] = s
+ * local, start: fp32 [segments][elems]; coef fp32 [elems]; x fp32 [segments][elems / group]. */
+int pcb_state_chain(const float* local, float* start, float* state, int64_t slot_stride, const int32_t* chains, int32_t n_chains,
+                    const float* coef, const float* x, int32_t elems, int32_t group, void* stream);
 
 #ifdef __cplusplus
 }

@@ -96,8 +96,13 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
 #pragma unroll
     for (int vb = 0; vb < VB; ++vb) o[vb] = f4{0.f, 0.f, 0.f, 0.f};
 
-    const int kb_lo = a.window > 0 ? (pos0 - a.window + 1 > 0 ? (pos0 - a.window + 1) / 32 : 0) : 0;
-    const int kb_hi = last / 32;
+    int kb_lo = a.window > 0 ? (pos0 - a.window + 1 > 0 ? (pos0 - a.window + 1) / 32 : 0) : 0;
+    int kb_hi = last / 32;
+    if (a.n_splits > 1) {                                   // this workgroup's run of the key blocks (it may be empty)
+        const int per = (kb_hi - kb_lo + a.n_splits) / a.n_splits;
+        kb_lo += (int)blockIdx.z * per;
+        kb_hi = kb_lo + per - 1 < kb_hi ? kb_lo + per - 1 : kb_hi;
+    }
     for (int kb = kb_lo + wave; kb <= kb_hi; kb += AW) {
         float s[8];
 #pragma unroll
@@ -188,6 +193,18 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
             for (int r = 0; r < 4; ++r) o[vb][r] += fw * red_o[w][(vb * 4 + r) * 64 + lane];
     }
     if (c >= rows) return;
+    if (a.n_splits > 1) {
+        float* pp = a.part + ((qrow * a.H + h) * a.n_splits + blockIdx.z) * (int64_t)(vdim + 2);
+        if (g == 0) pp[vdim] = mm, pp[vdim + 1] = lt;
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int col = vb * 16 + 4 * g + r;
+                if (col < vdim) pp[col] = o[vb][r];
+            }
+        return;
+    }
     const float inv = 1.0f / lt;
     E* op = (E*)a.out + qrow * a.ldo + (int64_t)h * vdim;
     const E* gp = a.gate ? (const E*)a.gate + qrow * a.ldg + (int64_t)h * vdim : nullptr;
@@ -204,9 +221,34 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
         }
 }
 
+// one workgroup per (tile, head): the runs' partial results of each query are rescaled to their common maximum and summed
+template <typename E>
+__global__ __launch_bounds__(256) void attn_merge_kernel(pcb_attn_softmax_args a) {
+    const int32_t* tile = a.tiles + 4 * blockIdx.x;
+    const int rows = tile[2], row0 = tile[3], h = blockIdx.y, vdim = a.vdim, Z = a.n_splits;
+    const float NEG = -__builtin_inff();
+    for (int i = threadIdx.x; i < rows * vdim; i += 256) {
+        const int64_t qrow = row0 + i / vdim;
+        const int col = i % vdim;
+        const float* pp = a.part + (qrow * a.H + h) * Z * (int64_t)(vdim + 2);
+        float mm = NEG;
+        for (int z = 0; z < Z; ++z) mm = fmaxf(mm, pp[z * (vdim + 2) + vdim]);
+        const float m_use = mm == NEG ? 0.0f : mm;
+        float l = 0.0f, o = 0.0f;
+        for (int z = 0; z < Z; ++z) {
+            const float f = expf(pp[z * (vdim + 2) + vdim] - m_use);
+            l += f * pp[z * (vdim + 2) + vdim + 1];
+            o += f * pp[z * (vdim + 2) + col];
+        }
+        float v = o / l;
+        if (a.gate) v *= to_f32(((const E*)a.gate)[qrow * a.ldg + (int64_t)h * vdim + col]);
+        ((E*)a.out)[qrow * a.ldo + (int64_t)h * vdim + col] = from_f32<E>(v);
+    }
+}
+
 template <typename E>
 int dispatch(const pcb_attn_softmax_args& a, hipStream_t stream) {
-    const dim3 grid(a.n_tiles, a.H), block(64 * AW);
+    const dim3 grid(a.n_tiles, a.H, a.n_splits > 1 ? a.n_splits : 1), block(64 * AW);
     const int big = a.dim > a.vdim ? a.dim : a.vdim;
     if (big <= 64)
         hipLaunchKernelGGL((attn_softmax_kernel<E, 2, 4>), grid, block, 0, stream, a);
@@ -214,6 +256,7 @@ int dispatch(const pcb_attn_softmax_args& a, hipStream_t stream) {
         hipLaunchKernelGGL((attn_softmax_kernel<E, 4, 8>), grid, block, 0, stream, a);
     else
         hipLaunchKernelGGL((attn_softmax_kernel<E, 8, 16>), grid, block, 0, stream, a);
+    if (a.n_splits > 1) hipLaunchKernelGGL(attn_merge_kernel<E>, dim3(a.n_tiles, a.H), dim3(256), 0, stream, a);
     return pcb_check_launch("attn_softmax_kernel");
 }
 
@@ -229,5 +272,6 @@ PCB_EXPORT int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream) {
     if (a->n_tiles == 0) return PCB_OK;
     PCB_REQUIRE(a->q && a->tiles && a->kcache && a->vcache && a->out && (!a->gate || a->ldg >= (int64_t)a->H * a->vdim), PCB_ERR_ARG,
                 "pcb_attn_softmax: null pointer");
+    PCB_REQUIRE(a->n_splits <= 1 || (a->part && a->n_splits <= 64), PCB_ERR_ARG, "pcb_attn_softmax: up to 64 runs, with their scratch");
     return a->dtype == PCB_BF16 ? dispatch<pcb::bf16_t>(*a, (hipStream_t)stream) : dispatch<float>(*a, (hipStream_t)stream);
 }

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(64) void decay_attn_kernel(pcb_decay_attn_args a) {
             vv[e] = (j < n && v_ok) ? to_f32(V[(r0 + j) * a.ldv + vcol]) : 0.0f;
             ot = mma4(vv[e], wt[e], ot);
         }
-        if (t_ok) {
+        if (t_ok && a.out) {
             float* op = a.out + (r0 + c) * a.ldo + (int64_t)h * vdim + blockIdx.z * 16;
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -224,8 +224,10 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(pcb_selective_scan_
         }
     };
     if (count > 0) fetch(0);
+    float dsum = 0.0f;
     for (int t = 0; t < count; ++t) {
         const float dt = dt_n, xv = x_n, zv = z_n;
+        dsum += dt;
         float Bc[NPL], Cc[NPL];
 #pragma unroll
         for (int i = 0; i < NPL; ++i) Bc[i] = B_n[i], Cc[i] = C_n[i];
@@ -239,18 +241,38 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(pcb_selective_scan_
         }
         y += __shfl_xor(y, 1, 64);
         y += __shfl_xor(y, 2, 64);
-        if (sub == 0 && ok) {
+        if (sub == 0 && ok && out) {
             y += Dv * xv;
             if (z) y *= zv / (1.0f + expf(-zv));
             out[(int64_t)(row0 + t) * a.ldo + ch] = from_f32<E>(y);
         }
     }
     if (!ok) return;
+    if (a.dt_sum && sub == 0) a.dt_sum[(int64_t)blockIdx.x * C + ch] = dsum;
 #pragma unroll
     for (int i = 0; i < NPL; ++i) {
         const int n = sub + 4 * i;
         if (n < N) st[n] = S[i];
     }
+}
+
+// ---- chaining the segments of a long prefill ----------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void state_chain_kernel(const float* __restrict__ local, float* __restrict__ start, float* __restrict__ state,
+                                                          int64_t slot_stride, const int32_t* __restrict__ chains,
+                                                          const float* __restrict__ coef, const float* __restrict__ x, int elems, int group) {
+    const int32_t* ch = chains + 4 * blockIdx.x;
+    const int slot = ch[0], pos0 = ch[1], g0 = ch[2], ng = ch[3];
+    const int e = blockIdx.y * 256 + threadIdx.x;
+    if (e >= elems) return;
+    const int groups = elems / group;
+    float* st = state + (int64_t)slot * slot_stride + e;
+    float s = pos0 > 0 ? *st : 0.0f;
+    const float cf = coef[e];
+    for (int g = g0; g < g0 + ng; ++g) {
+        start[(int64_t)g * elems + e] = s;
+        s = expf(cf * x[(int64_t)g * groups + e / group]) * s + local[(int64_t)g * elems + e];
+    }
+    *st = s;
 }
 
 template <typename E>
@@ -273,11 +295,11 @@ PCB_EXPORT int pcb_decay_attn(const pcb_decay_attn_args* a, void* stream) {
     PCB_REQUIRE(a && a->struct_bytes == sizeof(pcb_decay_attn_args), PCB_ERR_ARG, "pcb_decay_attn: struct size mismatch");
     PCB_REQUIRE(a->dtype == PCB_BF16 || a->dtype == PCB_F32, PCB_ERR_ARG, "pcb_decay_attn: unknown dtype");
     PCB_REQUIRE(a->n_reqs >= 0 && a->H > 0 && a->dim > 0 && a->dim <= 256 && a->vdim > 0 && a->ldq >= (int64_t)a->H * a->dim &&
-                    a->ldk >= (int64_t)a->H * a->dim && a->ldv >= (int64_t)a->H * a->vdim && a->ldo >= (int64_t)a->H * a->vdim &&
+                    a->ldk >= (int64_t)a->H * a->dim && a->ldv >= (int64_t)a->H * a->vdim && (!a->out || a->ldo >= (int64_t)a->H * a->vdim) &&
                     a->slot_stride >= (int64_t)a->H * a->dim * a->vdim && pcb_ceil_div(a->vdim, 16) <= 65535 && a->H <= 65535,
                 PCB_ERR_ARG, "pcb_decay_attn: bad sizes (key size up to 256)");
     if (a->n_reqs == 0) return PCB_OK;
-    PCB_REQUIRE(a->q && a->k && a->v && a->reqs && a->state && a->decay && a->out, PCB_ERR_ARG, "pcb_decay_attn: null pointer");
+    PCB_REQUIRE(a->q && a->k && a->v && a->reqs && a->state && a->decay, PCB_ERR_ARG, "pcb_decay_attn: null pointer");
     return a->dtype == PCB_BF16 ? launch_decay<pcb::bf16_t>(*a, (hipStream_t)stream) : launch_decay<float>(*a, (hipStream_t)stream);
 }
 
@@ -321,9 +343,20 @@ PCB_EXPORT int pcb_selective_scan(const pcb_selective_scan_args* a, void* stream
     PCB_REQUIRE(a && a->struct_bytes == sizeof(pcb_selective_scan_args), PCB_ERR_ARG, "pcb_selective_scan: struct size mismatch");
     PCB_REQUIRE(a->dtype == PCB_BF16 || a->dtype == PCB_F32, PCB_ERR_ARG, "pcb_selective_scan: unknown dtype");
     PCB_REQUIRE(a->n_reqs >= 0 && a->C > 0 && a->N > 0 && a->N <= 256 && a->ldx >= a->C && a->lddt >= a->C && a->ldbc >= a->N &&
-                    a->ldo >= a->C && (!a->z || a->ldz >= a->C) && a->slot_stride >= (int64_t)a->C * a->N,
+                    (!a->out || a->ldo >= a->C) && (!a->z || a->ldz >= a->C) && a->slot_stride >= (int64_t)a->C * a->N,
                 PCB_ERR_ARG, "pcb_selective_scan: bad sizes (up to 256 states per channel)");
     if (a->n_reqs == 0) return PCB_OK;
-    PCB_REQUIRE(a->x && a->dt && a->B && a->Cm && a->A && a->reqs && a->state && a->out, PCB_ERR_ARG, "pcb_selective_scan: null pointer");
+    PCB_REQUIRE(a->x && a->dt && a->B && a->Cm && a->A && a->reqs && a->state, PCB_ERR_ARG, "pcb_selective_scan: null pointer");
     return a->dtype == PCB_BF16 ? launch_scan<pcb::bf16_t>(*a, (hipStream_t)stream) : launch_scan<float>(*a, (hipStream_t)stream);
+}
+
+PCB_EXPORT int pcb_state_chain(const float* local, float* start, float* state, int64_t slot_stride, const int32_t* chains, int32_t n_chains,
+                               const float* coef, const float* x, int32_t elems, int32_t group, void* stream) {
+    PCB_REQUIRE(n_chains >= 0 && elems > 0 && group > 0 && elems % group == 0 && slot_stride >= elems && pcb_ceil_div(elems, 256) <= 65535,
+                PCB_ERR_ARG, "pcb_state_chain: bad sizes");
+    if (n_chains == 0) return PCB_OK;
+    PCB_REQUIRE(local && start && state && chains && coef && x, PCB_ERR_ARG, "pcb_state_chain: null pointer");
+    hipLaunchKernelGGL(state_chain_kernel, dim3(n_chains, pcb_ceil_div(elems, 256)), dim3(256), 0, (hipStream_t)stream, local, start, state,
+                       slot_stride, chains, coef, x, elems, group);
+    return pcb_check_launch("state_chain_kernel");
 }

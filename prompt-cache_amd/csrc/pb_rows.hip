@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256) void embed_pos_rows_kernel(const E* __restrict
 constexpr int MAX_STREAMS = 8;
 
 template <typename E>
-__global__ __launch_bounds__(256) void hyper_norm_kernel(pcb_hyper_norm_args a) {
+__global__ __launch_bounds__(1024) void hyper_norm_kernel(pcb_hyper_norm_args a) {
     extern __shared__ float row[];          // RMS only: the row between the sum and the norm
     __shared__ float red[16];
     __shared__ float coef[MAX_STREAMS * MAX_STREAMS + 2 * MAX_STREAMS];
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(256) void hyper_norm_kernel(pcb_hyper_norm_args a) 
     const float alpha = a.norm == PCB_NORM_DYT ? a.alpha[0] : 0.0f;
     float ss[1] = {0.0f};
     E* o = (E*)a.out;
-    for (int c = threadIdx.x; c < W; c += 256) {
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
         float x[MAX_STREAMS];
 #pragma unroll
         for (int s = 0; s < MAX_STREAMS; ++s) x[s] = s < S ? a.streams[s * a.stream_stride + src * W + c] : 0.0f;
@@ -346,7 +346,7 @@ __global__ __launch_bounds__(256) void hyper_norm_kernel(pcb_hyper_norm_args a) 
     if (o && a.norm == PCB_NORM_RMS) {
         block_sum<1>(ss, red);
         const float inv = 1.0f / sqrtf(ss[0] / (float)W + a.eps);
-        for (int c = threadIdx.x; c < W; c += 256) o[(int64_t)r * W + c] = from_f32<E>(row[c] * inv * a.gain[c]);
+        for (int c = threadIdx.x; c < W; c += blockDim.x) o[(int64_t)r * W + c] = from_f32<E>(row[c] * inv * a.gain[c]);
     }
 }
 
@@ -507,10 +507,12 @@ PCB_EXPORT int pcb_hyper_norm(const pcb_hyper_norm_args* a, void* stream) {
                 "pcb_hyper_norm: the norm needs its gain (and alpha)");
     PCB_REQUIRE(a->norm != PCB_NORM_RMS || a->width <= 16384, PCB_ERR_ARG, "pcb_hyper_norm: width <= 16384 with the RMS norm");
     const size_t lds = a->norm == PCB_NORM_RMS && a->out ? (size_t)a->width * sizeof(float) : 0;
+    // few rows: a row's columns are spread over up to 1024 threads (the loads of a thread's columns are a dependent chain)
+    const dim3 threads(a->n_rows <= 512 && a->width > 1024 ? 1024 : 256);
     if (a->dtype == PCB_BF16)
-        hipLaunchKernelGGL(hyper_norm_kernel<bf16_t>, dim3(a->n_rows), dim3(256), lds, (hipStream_t)stream, *a);
+        hipLaunchKernelGGL(hyper_norm_kernel<bf16_t>, dim3(a->n_rows), threads, lds, (hipStream_t)stream, *a);
     else
-        hipLaunchKernelGGL(hyper_norm_kernel<float>, dim3(a->n_rows), dim3(256), lds, (hipStream_t)stream, *a);
+        hipLaunchKernelGGL(hyper_norm_kernel<float>, dim3(a->n_rows), threads, lds, (hipStream_t)stream, *a);
     return pcb_check_launch("hyper_norm_kernel");
 }
 

@@ -70,7 +70,7 @@ class AttnSoftmaxArgs(C.Structure):
                 ("q", _vp), ("ldq", _i64), ("q_scale", _vp), ("tiles", _vp), ("n_tiles", _i32),
                 ("kcache", _vp), ("vcache", _vp), ("slot_stride", _i64), ("head_stride", _i64), ("row_stride", _i64),
                 ("H", _i32), ("Hkv", _i32), ("dim", _i32), ("vdim", _i32), ("scale", _f32), ("window", _i32),
-                ("gate", _vp), ("ldg", _i64), ("out", _vp), ("ldo", _i64)]
+                ("gate", _vp), ("ldg", _i64), ("out", _vp), ("ldo", _i64), ("n_splits", _i32), ("part", _vp)]
 
 
 class DecayAttnArgs(C.Structure):
@@ -86,7 +86,7 @@ class SelectiveScanArgs(C.Structure):
     _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
                 ("x", _vp), ("ldx", _i64), ("dt", _vp), ("lddt", _i64), ("B", _vp), ("Cm", _vp), ("ldbc", _i64),
                 ("z", _vp), ("ldz", _i64), ("A", _vp), ("D", _vp), ("reqs", _vp), ("n_reqs", _i32),
-                ("state", _vp), ("slot_stride", _i64), ("C", _i32), ("N", _i32), ("out", _vp), ("ldo", _i64)]
+                ("state", _vp), ("slot_stride", _i64), ("C", _i32), ("N", _i32), ("out", _vp), ("ldo", _i64), ("dt_sum", _vp)]
 
 
 # name -> (restype, argtypes); mirrors include/promptcache_blocks.h one to one
@@ -112,6 +112,7 @@ SIGNATURES = {
     "pcb_causal_conv": (C.c_int, [_vp, _i64, _vp, _vp, _i32, _i32, _vp, _vp, _i64, _vp, _i64, _i32, _i32, _i32, _vp]),
     "pcb_conv_state_update": (C.c_int, [_vp, _i64, _i32, _vp, _i32, _vp, _i64, _i32, _i32, _vp]),
     "pcb_selective_scan": (C.c_int, [C.POINTER(SelectiveScanArgs), _vp]),
+    "pcb_state_chain": (C.c_int, [_vp, _vp, _vp, _i64, _vp, _i32, _vp, _vp, _i32, _i32, _vp]),
 }
 
 
@@ -383,9 +384,12 @@ def moe_mix(pair_out: torch.Tensor, expert: torch.Tensor, weight: torch.Tensor, 
 
 def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, kcache: torch.Tensor, v_offset: int, slot_stride: int,
                  head_stride: int, row_stride: int, H: int, Hkv: int, dim: int, vdim: int, scale: float, out: torch.Tensor, *,
-                 q_scale: Optional[torch.Tensor] = None, window: int = 0, gate: Optional[torch.Tensor] = None, ldg: int = 0) -> None:
+                 q_scale: Optional[torch.Tensor] = None, window: int = 0, gate: Optional[torch.Tensor] = None, ldg: int = 0,
+                 n_splits: int = 1, part: Optional[torch.Tensor] = None) -> None:
     """``q``: E rows (row stride ``ldq``, head h at column h * dim); ``kcache``: the plane that holds the keys, the values
-    ``v_offset`` elements behind them; ``gate``: E rows of stride ``ldg``; ``out`` E [rows, H * vdim]."""
+    ``v_offset`` elements behind them; ``gate``: E rows of stride ``ldg``; ``out`` E [rows, H * vdim].  ``n_splits`` > 1: each
+    (tile, head) runs as that many workgroups over runs of the keys, merged by a second launch; ``part``: fp32 scratch of
+    ``attn_softmax_part(rows, H, n_splits, vdim)`` floats."""
     _want(tiles, torch.int32, "attn_softmax tiles"); _want(q_scale, torch.float32, "attn_softmax q_scale")
     assert q.dtype == kcache.dtype == out.dtype and out.is_contiguous() and kcache.is_cuda and q.is_cuda
     assert tiles.numel() >= 4 * n_tiles and out.shape[-1] == H * vdim and ldq >= H * dim
@@ -393,20 +397,27 @@ def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, k
     es = kcache.element_size()
     a = AttnSoftmaxArgs(C.sizeof(AttnSoftmaxArgs), _code(q), _p(q), ldq, _p(q_scale), _p(tiles), n_tiles, _p(kcache),
                         kcache.data_ptr() + v_offset * es, slot_stride, head_stride, row_stride, H, Hkv, dim, vdim, float(scale),
-                        int(window), _p(gate), ldg, _p(out), out.shape[-1])
+                        int(window), _p(gate), ldg, _p(out), out.shape[-1], int(n_splits), _p(part))
+    if n_splits > 1:
+        _want(part, torch.float32, "attn_softmax part")
+        assert part.numel() >= attn_softmax_part(out.shape[0], H, n_splits, vdim)
     check(load().pcb_attn_softmax(C.byref(a), _stream()), "pcb_attn_softmax")
 
 
+def attn_softmax_part(rows: int, H: int, n_splits: int, vdim: int) -> int:
+    return rows * H * n_splits * (vdim + 2)
+
+
 def decay_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ld: int, reqs: torch.Tensor, n_reqs: int, state: torch.Tensor,
-               decay: torch.Tensor, H: int, dim: int, vdim: int, out: torch.Tensor) -> None:
+               decay: torch.Tensor, H: int, dim: int, vdim: int, out: Optional[torch.Tensor]) -> None:
     """``q``, ``k``, ``v``: column blocks (row stride ``ld``) of one E matrix; ``state`` fp32 [slots, H, dim, vdim]; ``out`` fp32
-    [rows, H * vdim]."""
+    [rows, H * vdim], or None: only the states move."""
     _want(reqs, torch.int32, "decay_attn reqs"); _want(state, torch.float32, "decay_attn state"); _want(decay, torch.float32, "decay_attn decay")
     _want(out, torch.float32, "decay_attn out")
     assert q.dtype == k.dtype == v.dtype and q.is_cuda and reqs.numel() >= 4 * n_reqs and decay.numel() == H
-    assert tuple(state.shape[1:]) == (H, dim, vdim) and out.shape[-1] == H * vdim
+    assert tuple(state.shape[1:]) == (H, dim, vdim) and (out is None or out.shape[-1] == H * vdim)
     a = DecayAttnArgs(C.sizeof(DecayAttnArgs), _code(q), _p(q), _p(k), _p(v), ld, ld, ld, _p(reqs), n_reqs, _p(state), H * dim * vdim,
-                      _p(decay), H, dim, vdim, _p(out), out.shape[-1])
+                      _p(decay), H, dim, vdim, _p(out), H * vdim)
     check(load().pcb_decay_attn(C.byref(a), _stream()), "pcb_decay_attn")
 
 
@@ -430,16 +441,36 @@ def conv_state_update(x: torch.Tensor, ldx: int, reqs: torch.Tensor, n_reqs: int
 
 
 def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, z: Optional[torch.Tensor], ldz: int, A: torch.Tensor,
-                   D: Optional[torch.Tensor], reqs: torch.Tensor, n_reqs: int, state: torch.Tensor, out: torch.Tensor) -> None:
+                   D: Optional[torch.Tensor], reqs: torch.Tensor, n_reqs: int, state: torch.Tensor, out: Optional[torch.Tensor],
+                   dt_sum: Optional[torch.Tensor] = None) -> None:
     """``x`` E [rows, C]; ``dt`` fp32 [rows, C]; ``bc`` fp32 [rows, 2 N] = B | C; ``z`` E rows of stride ``ldz``; ``A`` fp32 [C, N];
-    ``state`` fp32 [slots, C, N]; ``out`` E [rows, C]."""
+    ``state`` fp32 [slots, C, N]; ``out`` E [rows, C], or None: only the states move; ``dt_sum`` fp32 [n_reqs, C]: each request's
+    sum of dt."""
     C_, N = A.shape
     for t, nm in ((dt, "dt"), (bc, "bc"), (A, "A"), (D, "D"), (state, "state")):
         _want(t, torch.float32, "selective_scan " + nm)
     _want(reqs, torch.int32, "selective_scan reqs")
-    assert x.dtype == out.dtype and x.is_contiguous() and out.is_contiguous() and x.shape[-1] == C_ == out.shape[-1] == dt.shape[-1]
+    assert x.is_contiguous() and x.shape[-1] == C_ == dt.shape[-1]
+    assert out is None or (x.dtype == out.dtype and out.is_contiguous() and out.shape[-1] == C_)
     assert bc.shape[-1] == 2 * N and tuple(state.shape[1:]) == (C_, N) and reqs.numel() >= 4 * n_reqs
     assert z is None or (z.dtype == x.dtype and ldz >= C_)
+    _want(dt_sum, torch.float32, "selective_scan dt_sum")
+    assert dt_sum is None or dt_sum.numel() >= n_reqs * C_
     a = SelectiveScanArgs(C.sizeof(SelectiveScanArgs), _code(x), _p(x), C_, _p(dt), C_, _p(bc), bc.data_ptr() + 4 * N, 2 * N, _p(z), ldz,
-                          _p(A), _p(D), _p(reqs), n_reqs, _p(state), C_ * N, C_, N, _p(out), C_)
+                          _p(A), _p(D), _p(reqs), n_reqs, _p(state), C_ * N, C_, N, _p(out), C_, _p(dt_sum))
     check(load().pcb_selective_scan(C.byref(a), _stream()), "pcb_selective_scan")
+
+
+def state_chain(local: torch.Tensor, start: torch.Tensor, state: torch.Tensor, chains: torch.Tensor, n_chains: int, coef: torch.Tensor,
+                x: torch.Tensor, group: int) -> None:
+    """``local``, ``start`` fp32 [segments, elems]; ``state`` fp32 [slots, ...elems]; ``chains`` int32 {slot, first position, first
+    segment, segments} x n_chains; ``coef`` fp32 [elems]; ``x`` fp32 [segments, elems / group]."""
+    for t, nm in ((local, "local"), (start, "start"), (state, "state"), (coef, "coef"), (x, "x")):
+        _want(t, torch.float32, "state_chain " + nm)
+    _want(chains, torch.int32, "state_chain chains")
+    elems = coef.numel()
+    n_seg = local.shape[0]
+    assert local.numel() == n_seg * elems == start.numel() and state[0].numel() == elems and chains.numel() >= 4 * n_chains
+    assert elems % group == 0 and x.numel() >= n_seg * (elems // group)
+    check(load().pcb_state_chain(_p(local), _p(start), _p(state), elems, _p(chains), n_chains, _p(coef), _p(x), elems, group, _stream()),
+          "pcb_state_chain")

@@ -46,6 +46,8 @@ from .slot_model import SlotKV, SlotModel  # noqa: F401
 
 class DibizenHIP(SlotModel):
     GRAPH_MAX_ROWS = 64
+    SEGMENT = 128           # a step that brings a request more tokens than this runs its recurrent mixers segment-parallel
+    MAX_SEGMENTS = 64       # (segments grow beyond SEGMENT tokens rather than exceed this many per request)
 
     def __init__(self, shape: DibizenShape, weights: Dict[str, torch.Tensor], device="cuda:0", dtype=torch.bfloat16,
                  decode_headroom: int = 256):
@@ -87,6 +89,9 @@ class DibizenHIP(SlotModel):
                     raise ValueError(f"layer {i}: lightning heads take up to 256 key columns (got {l.dim})")
                 ent.update(w_in=torch.cat([e(m + "q"), e(m + "k"), e(m + "v"), e(m + "g")], dim=0).contiguous(), wo=e(m + "o"),
                            gain=f(m + "norm"), decay=torch.tensor(l.decay, dtype=torch.float32, device=dev))
+                # ln(decay) per state element: the factor a state takes over a segment of n tokens is exp(n ln(decay))
+                lnd = torch.tensor([math.log(d) if d > 0 else -math.inf for d in l.decay], dtype=torch.float32, device=dev)
+                ent["ln_decay"] = lnd.view(-1, 1).expand(l.heads, l.dim * l.vdim).reshape(-1).contiguous()
             elif l.kind == "attention":
                 if max(l.dim, l.vdim) > 256:
                     raise ValueError(f"layer {i}: attention heads take up to 256 columns (got {l.dim} / {l.vdim})")
@@ -187,19 +192,36 @@ class DibizenHIP(SlotModel):
             picked = [b for b, ws in enumerate(want) for _ in ws]
         want_rows = np.arange(T, dtype=np.int32) if graphed else \
             np.asarray([int(row0[b]) + int(w) for b, ws in enumerate(want) for w in ws], dtype=np.int32)
+        # segments of the recurrent mixers' prefill (only when some request brings more than SEGMENT tokens)
+        seg_a = seg_c = chains = np.zeros((0, 4), np.int32)
+        seg_n = np.zeros(0, np.float32)
+        if max(counts) > self.SEGMENT and any(l.kind != "attention" for l in self.config.layers):
+            seg = max(self.SEGMENT, -(-max(counts) // self.MAX_SEGMENTS))
+            seg = -(-seg // 16) * 16
+            sa, ch = [], []
+            for b, (s, st, c) in enumerate(zip(slots, starts, counts)):
+                ch.append((s, st, len(sa), -(-c // seg)))
+                sa += [(len(sa) + k, 0, min(seg, c - q), int(row0[b]) + q) for k, q in enumerate(range(0, c, seg))]
+            seg_a = np.asarray(sa, dtype=np.int32)
+            seg_c = seg_a.copy()
+            seg_c[:, 1] = 1                                 # the second pass starts every segment from a state that was put there
+            chains = np.asarray(ch, dtype=np.int32)
+            seg_n = seg_a[:, 2].astype(np.float32)
         temps = np.stack([1.0 + coef * np.log(np.floor((row_pos + 1) / every) + 1.0) for coef, every in self._temps]).astype(np.float32) \
             if self._temps else np.zeros((0, T), np.float32)
         offs = np.stack([row_slot * (g * arena.cap * d) + row_pos * d for g, d in self._sigs]) if self._sigs else np.zeros((0, T), np.int64)
         # one block: int32 tables, then fp32 temperatures, then int64 cache offsets
-        parts32 = [ids, row_pos.astype(np.int32), meta.reshape(-1), reqs.reshape(-1), tiles.reshape(-1), want_rows]
+        parts32 = [ids, row_pos.astype(np.int32), meta.reshape(-1), reqs.reshape(-1), tiles.reshape(-1), want_rows, seg_a.reshape(-1),
+                   seg_c.reshape(-1), chains.reshape(-1)]
         n32 = sum(p.size for p in parts32)
-        nf = temps.size
+        nf = temps.size + seg_n.size
         o64 = ((n32 + nf) * 4 + 7) // 8 * 8
         blob = np.empty(o64 + offs.size * 8 + 8, dtype=np.uint8)
         blob[:n32 * 4].view(np.int32)[:] = np.concatenate(parts32)
-        blob[n32 * 4:(n32 + nf) * 4].view(np.float32)[:] = temps.reshape(-1)
+        blob[n32 * 4:(n32 + nf) * 4].view(np.float32)[:] = np.concatenate([temps.reshape(-1), seg_n])
         blob[o64:o64 + offs.size * 8].view(np.int64)[:] = offs.reshape(-1)
-        dims = dict(T=T, R=R, n_tiles=tiles.shape[0], n_want=int(want_rows.size), n32=n32, o64=o64)
+        dims = dict(T=T, R=R, n_tiles=tiles.shape[0], n_want=int(want_rows.size), n32=n32, o64=o64, n_seg=seg_a.shape[0],
+                    n_chains=chains.shape[0])
         res = self._decode_graphed(arena, blob, dims) if graphed else None
         if res is None:
             dblob = torch.from_numpy(blob).to(dev)
@@ -212,14 +234,18 @@ class DibizenHIP(SlotModel):
         return res
 
     def _tables(self, dblob, d):
-        T, R, nt, nw = d["T"], d["R"], d["n_tiles"], d["n_want"]
+        T, R, nt, nw, ns = d["T"], d["R"], d["n_tiles"], d["n_want"], d["n_seg"]
         i32 = dblob[:d["n32"] * 4].view(torch.int32)
         at, out = 0, {}
-        for name, n in (("ids", T), ("pos", T), ("meta", 4 * T), ("reqs", 4 * R), ("tiles", 4 * nt), ("want", nw)):
+        for name, n in (("ids", T), ("pos", T), ("meta", 4 * T), ("reqs", 4 * R), ("tiles", 4 * nt), ("want", nw), ("seg_a", 4 * ns),
+                        ("seg_c", 4 * ns), ("chains", 4 * d["n_chains"])):
             out[name] = i32[at:at + n]
             at += n
         nf = len(self._temps) * T
-        out["temps"] = dblob[d["n32"] * 4:(d["n32"] + nf) * 4].view(torch.float32).view(len(self._temps), T)
+        f32 = dblob[d["n32"] * 4:(d["n32"] + nf + ns) * 4].view(torch.float32)
+        out["temps"] = f32[:nf].view(len(self._temps), T)
+        out["seg_n"] = f32[nf:nf + ns]
+        out["n_seg"], out["n_chains"] = ns, d["n_chains"]
         out["offs"] = dblob[d["o64"]:d["o64"] + len(self._sigs) * T * 8].view(torch.int64).view(len(self._sigs), T)
         return out
 
@@ -279,7 +305,18 @@ class DibizenHIP(SlotModel):
         qkvg = self._mat("mix_in", T, N, self.dtype)
         B.linear(h, lw["w_in"], qkvg, M=T, act=B.ACT_SILU, act_split=2 * HD + HV, act2=B.ACT_SIGMOID)
         o = self._mat("mix_o32", T, HV, torch.float32)
-        B.decay_attn(qkvg, qkvg[:, HD:], qkvg[:, 2 * HD:], N, tb["reqs"], R, arena.states[i][0], lw["decay"], l.heads, l.dim, l.vdim, o)
+        state, ns = arena.states[i][0], tb["n_seg"]
+        q, k, v = qkvg, qkvg[:, HD:], qkvg[:, 2 * HD:]
+        if ns:
+            # every segment from a zero state (only the states move), the segments chained, then every segment from its start state
+            elems = l.heads * l.dim * l.vdim
+            local = self._scratch("seg_local", ns * elems, torch.float32)[:ns * elems].view(ns, l.heads, l.dim, l.vdim)
+            start = self._scratch("seg_start", ns * elems, torch.float32)[:ns * elems].view(ns, l.heads, l.dim, l.vdim)
+            B.decay_attn(q, k, v, N, tb["seg_a"], ns, local, lw["decay"], l.heads, l.dim, l.vdim, None)
+            B.state_chain(local, start, state, tb["chains"], tb["n_chains"], lw["ln_decay"], tb["seg_n"], elems)
+            B.decay_attn(q, k, v, N, tb["seg_c"], ns, start, lw["decay"], l.heads, l.dim, l.vdim, o)
+        else:
+            B.decay_attn(q, k, v, N, tb["reqs"], R, state, lw["decay"], l.heads, l.dim, l.vdim, o)
         on = self._mat("mix_out", T, HV, self.dtype)
         B.gated_norm(o, lw["gain"], qkvg[:, 2 * HD + HV:], N, on, self.config.norm_eps, T)
         B.linear(on, lw["wo"], y, M=T)
@@ -296,8 +333,11 @@ class DibizenHIP(SlotModel):
             B.linear(h, lw["w_in"], qg, M=T, act_split=HD, act2=B.ACT_SIGMOID)
         att = self._mat("mix_out", T, HV, self.dtype)
         temp = tb["temps"][self._temps.index((l.qt_coef, l.qt_every))] if l.qt_every else None
+        # few (tile, head) pairs cannot fill the chip: each is cut into runs of its keys (steps of few rows over long caches)
+        splits = 1 if n_tiles * l.heads >= 512 or arena.cap <= 256 else max(1, min(16, 1024 // (n_tiles * l.heads), arena.cap // 128))
+        part = self._scratch("attn_part", B.attn_softmax_part(T, l.heads, splits, l.vdim), torch.float32) if splits > 1 else None
         B.attn_softmax(qg, HD + HV, tb["tiles"], n_tiles, plane, l.dim, arena.slot_stride(src), arena.head_stride(src), dv, l.heads,
-                       l.kv_heads, l.dim, l.vdim, l.scale, att, q_scale=temp, gate=qg[:, HD:], ldg=HD + HV)
+                       l.kv_heads, l.dim, l.vdim, l.scale, att, q_scale=temp, gate=qg[:, HD:], ldg=HD + HV, n_splits=splits, part=part)
         B.linear(att, lw["wo"], y, M=T)
 
     def _mamba(self, arena, i, l, lw, h, y, tb, T, R):
@@ -315,7 +355,16 @@ class DibizenHIP(SlotModel):
         dt = self._mat("scan_dt", T, C, torch.float32)
         B.linear(low, lw["wdt"], dt, M=T, bias=lw["dt_b"], act=B.ACT_SOFTPLUS)
         ys = self._mat("scan_y", T, C, E)
-        B.selective_scan(xc, dt, bc, xz[:, C:], 2 * C, lw["A"], lw["D"], tb["reqs"], R, state, ys)
+        ns = tb["n_seg"]
+        if ns:
+            local = self._scratch("seg_local", ns * C * N, torch.float32)[:ns * C * N].view(ns, C, N)
+            start = self._scratch("seg_start", ns * C * N, torch.float32)[:ns * C * N].view(ns, C, N)
+            dsum = self._mat("seg_dt", ns, C, torch.float32)
+            B.selective_scan(xc, dt, bc, None, 0, lw["A"], None, tb["seg_a"], ns, local, None, dt_sum=dsum)
+            B.state_chain(local, start, state, tb["chains"], tb["n_chains"], lw["A"].view(-1), dsum, N)
+            B.selective_scan(xc, dt, bc, xz[:, C:], 2 * C, lw["A"], lw["D"], tb["seg_c"], ns, start, ys)
+        else:
+            B.selective_scan(xc, dt, bc, xz[:, C:], 2 * C, lw["A"], lw["D"], tb["reqs"], R, state, ys)
         B.linear(ys, lw["wo"], y, M=T)
 
     def _experts(self, l, lw, h, y, T):

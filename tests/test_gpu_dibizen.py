@@ -194,7 +194,7 @@ def test_router_select_and_moe_mix(E, top, groups, keep):
     assert rel(y, (w.unsqueeze(-1) * src).sum(dim=1)) < 1e-6
 
 
-def attention_case(dtype, H, G, D, Dv, lens, news, seed=0, boost=None):
+def attention_case(dtype, H, G, D, Dv, lens, news, seed=0, boost=None, splits=1):
     """``lens[b]`` keys of request b are in the cache (its slot b of a plane with interleaved key | value rows), the last
     ``news[b]`` of them belong to this step's queries.  Returns (kernel output, oracle output)."""
     cap, Bn = max(lens) + 3, len(lens)
@@ -214,8 +214,9 @@ def attention_case(dtype, H, G, D, Dv, lens, news, seed=0, boost=None):
             tiles.append((b, n - m + c, min(16, m - c), row0 + c))
         row0 += m
     out = torch.empty((T, H * Dv), dtype=dtype, device=DEV)
+    part = torch.empty(B().attn_softmax_part(T, H, splits, Dv), dtype=torch.float32, device=DEV) if splits > 1 else None
     B().attn_softmax(q, H * D + 5, dev_i32(tiles), len(tiles), plane, D, G * cap * (D + Dv), cap * (D + Dv), D + Dv, H, G, D, Dv, 0.3, out,
-                     q_scale=qs, gate=gate, ldg=H * Dv)
+                     q_scale=qs, gate=gate, ldg=H * Dv, n_splits=splits, part=part)
     want, row0 = [], 0
     for b, (n, m) in enumerate(zip(lens, news)):
         qq = q[row0:row0 + m, :H * D].to(F64).cpu().view(m, H, D) * qs[row0:row0 + m].to(F64).cpu().view(m, 1, 1)
@@ -235,10 +236,18 @@ def test_softmax_attention_alone(dtype, H, G, D, Dv):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("key", [0, 31, 32, 127, 128, 299])
-def test_softmax_attention_finds_a_far_key(dtype, key):
+@pytest.mark.parametrize("splits", [2, 5, 16])
+def test_softmax_attention_in_runs_of_the_keys(dtype, splits):
+    # more runs than some requests have key blocks: empty runs must drop out of the merge
+    got, want = attention_case(dtype, 4, 2, 48, 40, lens=[45, 700, 1, 32, 33, 257], news=[45, 1, 1, 17, 2, 1], seed=splits, splits=splits)
+    assert rel(got, want) < tol(dtype, 1e-5, 1.5e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("key,splits", [(0, 1), (31, 1), (32, 4), (127, 1), (128, 4), (299, 1), (299, 7)])
+def test_softmax_attention_finds_a_far_key(dtype, key, splits):
     # the last query's score for ONE key of 300 is raised far above the rest: its head's output must be that key's value
-    got, want = attention_case(dtype, 2, 1, 40, 24, lens=[300, 300], news=[1, 20], seed=3, boost=(1, key, 1, 60.0))
+    got, want = attention_case(dtype, 2, 1, 40, 24, lens=[300, 300], news=[1, 20], seed=3, boost=(1, key, 1, 60.0), splits=splits)
     assert rel(got, want) < tol(dtype, 1e-5, 1.5e-2)
     assert rel(got[-1, 24:], want[-1, 24:]) < tol(dtype, 1e-5, 1.5e-2)
 
@@ -368,6 +377,24 @@ def test_portions_of_a_prompt(cuts, dtype):
     s, w, m = model("mixed", dtype)
     t = toks(40, s.vocab_size, seed=7)
     assert rel(run_alone(m, t, cuts), O.forward(t, w, s)) < tol(dtype, 2e-5, 3e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["mixed", "odd"])
+def test_segmented_prefill_of_the_recurrent_mixers(name, dtype, monkeypatch):
+    # segments of 16 tokens: prompts of several ragged segments, a portion that continues a carried state, an unequal batch
+    s, w, m = model(name, dtype)
+    monkeypatch.setattr(m, "SEGMENT", 16)
+    t = toks(75, s.vocab_size, seed=3)
+    want = O.forward(t, w, s)
+    assert rel(run_alone(m, t), want) < tol(dtype, 2e-5, 3e-2)
+    assert rel(run_alone(m, t, [3, 40, 32]), want) < tol(dtype, 2e-5, 3e-2)
+    u = toks(17, s.vocab_size, seed=4)
+    ar = m.new_arena(2, 8)
+    got = m.forward_rows(ar, [ar.alloc(), ar.alloc()], [u, t], [list(range(17)), list(range(75))])
+    assert rel(got, torch.cat([O.forward(u, w, s), want])) < tol(dtype, 2e-5, 3e-2)
+    monkeypatch.setattr(m, "MAX_SEGMENTS", 2)              # longer segments rather than more of them
+    assert rel(run_alone(m, t), want) < tol(dtype, 2e-5, 3e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
