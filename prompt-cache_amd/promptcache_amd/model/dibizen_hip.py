@@ -46,7 +46,7 @@ from .slot_model import SlotKV, SlotModel  # noqa: F401
 
 class DibizenHIP(SlotModel):
     GRAPH_MAX_ROWS = 64
-    SEGMENT = 128           # a step that brings a request more tokens than this runs its recurrent mixers segment-parallel
+    SEGMENT = int(os.environ.get("PC_DZ_SEGMENT", "128"))   # a step that brings a request more tokens than this runs its recurrent mixers segment-parallel
     MAX_SEGMENTS = 64       # (segments grow beyond SEGMENT tokens rather than exceed this many per request)
 
     def __init__(self, shape: DibizenShape, weights: Dict[str, torch.Tensor], device="cuda:0", dtype=torch.bfloat16,
