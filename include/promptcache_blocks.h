@@ -103,7 +103,13 @@ typedef struct pcb_linear_args {
     const int64_t* row_off2;
     int32_t head_dim2;
     int64_t head_stride2;
-    int32_t act;       /* PCB_ACT_*: STORE only, applied to acc + bias before the store (not to the columns split off to y2) */
+    int32_t split_n3;  /* > 0 (STORE only): columns n >= split_n3 go to y3 instead, one element per (row, column) with the ROW index
+                          running fastest in memory: row m, column c = n - split_n3 at y3 + row_off3[m] + c * col_stride3 (a projection
+                          that appends its last part to a cache kept column by column) */
+    void* y3;
+    const int64_t* row_off3;
+    int64_t col_stride3;
+    int32_t act;       /* PCB_ACT_*: STORE only, applied to acc + bias before the store (not to the columns split off to y2 / y3) */
     int32_t act_split; /* > 0: columns n >= act_split take act2 instead of act */
     int32_t act2;
     float act_param;   /* PCB_ACT_SOFTCAP: the cap */
@@ -232,9 +238,11 @@ int pcb_moe_mix(const float* pair_out, const int32_t* expert, const float* weigh
 
 /* Causal softmax attention over a slot-addressed cache with separate keys and values.
  * Queries are flat rows; tile t = {slot, first query position, query rows (<= 16), first flat row} (int32 x 4, device).
- * Key j of kv head g of slot s: kcache + s * slot_stride + g * head_stride + j * row_stride (dim elements); its value at the same
- * offset from vcache (vdim elements) -- keys and values may interleave in one plane.  The cache already holds the queries' own
- * keys.  score = q_scale[row] * scale * q.k (q_scale null: 1); key j is seen by the query at position i iff j <= i and
+ * Key j of kv head g of slot s: kcache + s * slot_stride + g * head_stride + j * row_stride (dim elements).  Its value: row by row
+ * like the keys (v_cols = 0: vcache + s * v_slot_stride + g * v_head_stride + j * v_stride, vdim elements -- keys and values may
+ * interleave in one plane), or column by column (v_cols = 1: column c of key j at vcache + s * v_slot_stride + g * v_head_stride +
+ * c * v_stride + j; every column must be readable up to the next multiple of 32 keys, and v_stride a multiple of 8), which lets
+ * the value operand of the matrix cores be read with wide loads.  The cache already holds the queries' own keys and values.  score = q_scale[row] * scale * q.k (q_scale null: 1); key j is seen by the query at position i iff j <= i and
  * (window <= 0 or i - j < window).  The result (E [rows][ldo], head h at column h * vdim) is multiplied element-wise by
  * gate[row][..] (E, ldg) when given.  dim, vdim <= 256. */
 typedef struct pcb_attn_softmax_args {
@@ -248,6 +256,8 @@ typedef struct pcb_attn_softmax_args {
     const void* kcache;
     const void* vcache;
     int64_t slot_stride, head_stride, row_stride;
+    int64_t v_slot_stride, v_head_stride, v_stride;
+    int32_t v_cols;
     int32_t H, Hkv, dim, vdim;
     float scale;
     int32_t window;

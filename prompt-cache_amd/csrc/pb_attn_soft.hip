@@ -59,6 +59,39 @@ __device__ __forceinline__ Frag<float> load_v(const float* const (&rows)[8], int
     return f;
 }
 
+// the same operand from a cache kept column by column: `col` points at key 32 kb of the lane's value column; the lane's eight keys
+// are the two runs 4 g .. 4 g + 3 and 16 + 4 g .. 16 + 4 g + 3, one wide load each.  Keys past `valid` (counted from key 32 kb)
+// are replaced by zeros: what lies there need not be numbers.
+__device__ __forceinline__ Frag<bf16_t> load_v_cols(const bf16_t* col, int g, bool ok, int valid) {
+    Frag<bf16_t> f;
+    uint2 lo = uint2{0u, 0u}, hi = uint2{0u, 0u};
+    if (ok) {
+        lo = *reinterpret_cast<const uint2*>(col + 4 * g);
+        hi = *reinterpret_cast<const uint2*>(col + 16 + 4 * g);
+    }
+    if (valid < 32) {
+        const int a = valid - 4 * g, b = valid - 16 - 4 * g;      // how many of each run exist
+        lo.x &= a >= 2 ? 0xffffffffu : (a == 1 ? 0x0000ffffu : 0u);
+        lo.y &= a >= 4 ? 0xffffffffu : (a == 3 ? 0x0000ffffu : 0u);
+        hi.x &= b >= 2 ? 0xffffffffu : (b == 1 ? 0x0000ffffu : 0u);
+        hi.y &= b >= 4 ? 0xffffffffu : (b == 3 ? 0x0000ffffu : 0u);
+    }
+    f.v = u32x4{lo.x, lo.y, hi.x, hi.y};
+    return f;
+}
+__device__ __forceinline__ Frag<float> load_v_cols(const float* col, int g, bool ok, int valid) {
+    Frag<float> f;
+    float4 lo = float4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+    if (ok) {
+        lo = *reinterpret_cast<const float4*>(col + 4 * g);
+        hi = *reinterpret_cast<const float4*>(col + 16 + 4 * g);
+    }
+    const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f.v[e] = ((e < 4 ? 4 * g + e : 16 + 4 * g + e - 4) < valid) ? v[e] : 0.0f;
+    return f;
+}
+
 __device__ __forceinline__ f4 mma_p(const Frag<bf16_t>& v, const PFrag<bf16_t>& p, f4 c) {
     c = mma(v, p.hi, c);
     return mma(v, p.lo, c);
@@ -80,7 +113,7 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
     const int qpos = pos0 + qi;
     const int64_t qrow = row0 + qi;
     const E* K = (const E*)a.kcache + (int64_t)slot * a.slot_stride + (int64_t)hk * a.head_stride;
-    const E* V = (const E*)a.vcache + (int64_t)slot * a.slot_stride + (int64_t)hk * a.head_stride;
+    const E* V = (const E*)a.vcache + (int64_t)slot * a.v_slot_stride + (int64_t)hk * a.v_head_stride;
     const E* qp = (const E*)a.q + qrow * a.ldq + (int64_t)h * dim;
     constexpr int CE = 16 / sizeof(E);
     const bool qvec = ((uintptr_t)a.q % 16 == 0) && (a.ldq % CE == 0) && (dim % CE == 0);
@@ -143,13 +176,15 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
         for (int e = 0; e < 8; ++e) {
             int key = kb * 32 + (e < 4 ? 4 * g + e : 16 + 4 * g + e - 4);
             key = key > last ? last : key;
-            vrows[e] = V + (int64_t)key * a.row_stride;
+            vrows[e] = V + (int64_t)key * a.v_stride;
         }
+        const int v_valid = last + 1 - kb * 32;             // keys of this block that exist
 #pragma unroll
         for (int vb = 0; vb < VB; ++vb) {
             if (vb * 16 >= vdim) break;
             const int col = vb * 16 + c;
-            const Frag<E> vf = load_v(vrows, col, col < vdim);
+            const Frag<E> vf = a.v_cols ? load_v_cols(V + (int64_t)(col < vdim ? col : 0) * a.v_stride + kb * 32, g, col < vdim, v_valid)
+                                        : load_v(vrows, col, col < vdim);
             f4 t = o[vb];
 #pragma unroll
             for (int r = 0; r < 4; ++r) t[r] *= alpha;
@@ -267,8 +302,10 @@ PCB_EXPORT int pcb_attn_softmax(const pcb_attn_softmax_args* a, void* stream) {
     PCB_REQUIRE(a->dtype == PCB_BF16 || a->dtype == PCB_F32, PCB_ERR_ARG, "pcb_attn_softmax: unknown dtype");
     PCB_REQUIRE(a->n_tiles >= 0 && a->H > 0 && a->Hkv > 0 && a->H % a->Hkv == 0 && a->dim > 0 && a->dim <= 256 && a->vdim > 0 &&
                     a->vdim <= 256 && a->ldq >= (int64_t)a->H * a->dim && a->ldo >= (int64_t)a->H * a->vdim &&
-                    a->row_stride >= a->dim && a->row_stride >= a->vdim,
-                PCB_ERR_ARG, "pcb_attn_softmax: bad sizes (key and value sizes up to 256)");
+                    a->row_stride >= a->dim && (a->v_cols ? (a->v_stride % 8 == 0 && a->v_stride > 0 && (uintptr_t)a->vcache % 16 == 0 &&
+                                                             a->v_head_stride % 8 == 0 && a->v_slot_stride % 8 == 0)
+                                                          : a->v_stride >= a->vdim),
+                PCB_ERR_ARG, "pcb_attn_softmax: bad sizes (key and value sizes up to 256; a column-wise value cache in multiples of 8)");
     if (a->n_tiles == 0) return PCB_OK;
     PCB_REQUIRE(a->q && a->tiles && a->kcache && a->vcache && a->out && (!a->gate || a->ldg >= (int64_t)a->H * a->vdim), PCB_ERR_ARG,
                 "pcb_attn_softmax: null pointer");

@@ -59,13 +59,18 @@ __device__ __forceinline__ float apply_act(int act, float v, float param) {
 template <typename E, int EPI>
 __device__ __forceinline__ void emit(const pcb_linear_args& a, int m, int n, float acc, float acc2, float bv, float cs) {
     float v = acc + bv;
-    if (EPI == PCB_EPI_STORE && (a.act | a.act2) && !(a.split_n > 0 && n >= a.split_n))      // (the split-off part is stored as it is)
+    if (EPI == PCB_EPI_STORE && (a.act | a.act2) && !(a.split_n > 0 && n >= a.split_n) && !(a.split_n3 > 0 && n >= a.split_n3))
+        // (the split-off parts are stored as they are)
         v = apply_act((a.act_split > 0 && n >= a.act_split) ? a.act2 : a.act, v, a.act_param);
     if (EPI == PCB_EPI_SILU_MUL) v = acc / (1.0f + expf(-acc)) * acc2;
     if (EPI == PCB_EPI_SCALE_ADD) {
         float* y = (float*)a.y + (int64_t)m * a.ldy + n;
         const float b0 = a.base ? a.base[(int64_t)m * a.ldbase + n] : *y;
         *y = b0 + cs * v;
+        return;
+    }
+    if (a.split_n3 > 0 && n >= a.split_n3) {
+        ((E*)a.y3)[a.row_off3[m] + (int64_t)(n - a.split_n3) * a.col_stride3] = from_f32<E>(v);
         return;
     }
     if (a.split_n > 0 && n >= a.split_n) {
@@ -374,6 +379,9 @@ PCB_EXPORT int pcb_linear(const pcb_linear_args* a, void* stream) {
     PCB_REQUIRE(a->split_n == 0 || (a->epilogue == PCB_EPI_STORE && a->split_n > 0 && a->split_n < a->N && a->y2 && a->row_off2 &&
                                     a->head_dim2 > 0 && a->ldy >= a->split_n),
                 PCB_ERR_ARG, "pcb_linear: bad split destination");
-    PCB_REQUIRE(a->split_n > 0 || a->epilogue == PCB_EPI_SCALE_ADD || a->ldy >= a->N, PCB_ERR_ARG, "pcb_linear: ldy < N");
+    PCB_REQUIRE(a->split_n3 == 0 || (a->epilogue == PCB_EPI_STORE && a->split_n3 > a->split_n && a->split_n3 < a->N && a->y3 && a->row_off3 &&
+                                     a->col_stride3 > 0 && (a->split_n > 0 || a->ldy >= a->split_n3)),
+                PCB_ERR_ARG, "pcb_linear: bad column-wise destination");
+    PCB_REQUIRE(a->split_n > 0 || a->split_n3 > 0 || a->epilogue == PCB_EPI_SCALE_ADD || a->ldy >= a->N, PCB_ERR_ARG, "pcb_linear: ldy < N");
     return a->dtype == PCB_BF16 ? dispatch<pcb::bf16_t>(*a, (hipStream_t)stream) : dispatch<float>(*a, (hipStream_t)stream);
 }

@@ -41,6 +41,7 @@ class LinearArgs(C.Structure):
                 ("y", _vp), ("ldy", _i64), ("out_f32", _i32), ("row_dst", _vp),
                 ("base", _vp), ("ldbase", _i64), ("col_scale", _vp),
                 ("split_n", _i32), ("y2", _vp), ("row_off2", _vp), ("head_dim2", _i32), ("head_stride2", _i64),
+                ("split_n3", _i32), ("y3", _vp), ("row_off3", _vp), ("col_stride3", _i64),
                 ("act", _i32), ("act_split", _i32), ("act2", _i32), ("act_param", _f32)]
 
 
@@ -69,6 +70,7 @@ class AttnSoftmaxArgs(C.Structure):
     _fields_ = [("struct_bytes", C.c_uint32), ("dtype", _i32),
                 ("q", _vp), ("ldq", _i64), ("q_scale", _vp), ("tiles", _vp), ("n_tiles", _i32),
                 ("kcache", _vp), ("vcache", _vp), ("slot_stride", _i64), ("head_stride", _i64), ("row_stride", _i64),
+                ("v_slot_stride", _i64), ("v_head_stride", _i64), ("v_stride", _i64), ("v_cols", _i32),
                 ("H", _i32), ("Hkv", _i32), ("dim", _i32), ("vdim", _i32), ("scale", _f32), ("window", _i32),
                 ("gate", _vp), ("ldg", _i64), ("out", _vp), ("ldo", _i64), ("n_splits", _i32), ("part", _vp)]
 
@@ -201,7 +203,8 @@ def mix_norm(hist: torch.Tensor, n_streams: int, coef: Optional[torch.Tensor], g
 
 def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, M: int, epilogue: int = EPI_STORE, bias=None, w2=None,
            row_src=None, row_scale=None, group_off=None, n_groups: int = 0, row_dst=None, base=None, col_scale=None,
-           split_n: int = 0, y2=None, row_off2=None, head_dim2: int = 0, head_stride2: int = 0, act: int = ACT_NONE,
+           split_n: int = 0, y2=None, row_off2=None, head_dim2: int = 0, head_stride2: int = 0, split_n3: int = 0, y3=None,
+           row_off3=None, col_stride3: int = 0, act: int = ACT_NONE,
            act_split: int = 0, act2: int = ACT_NONE, act_param: float = 0.0, ldy: Optional[int] = None) -> None:
     """``w``: [N, K], or [groups, N, K] with ``group_off``.  ``x``: [rows, K] of the weights' element type.  ``act`` (and ``act2``
     from column ``act_split`` on): the element-wise function of a plain store.  ``ldy``: row stride of ``y`` when it is a
@@ -237,15 +240,18 @@ def linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, M: int, epilogu
             assert base.shape[-1] == N and base.shape[0] >= M
     else:
         assert y.is_contiguous() and (y.dtype == w.dtype or y.dtype == torch.float32)
-        cols = split_n if split_n else N
+        cols = split_n if split_n else (split_n3 if split_n3 else N)
         assert (y.shape[-1] == cols or (ldy is not None and ldy >= cols)) and (row_dst is not None or y.shape[0] >= M)
     if split_n:
         _want(row_off2, torch.int64, "linear row_off2")
         assert y2 is not None and y2.dtype == w.dtype and row_off2.numel() >= M and head_dim2 > 0
+    if split_n3:
+        _want(row_off3, torch.int64, "linear row_off3")
+        assert y3 is not None and y3.dtype == w.dtype and row_off3.numel() >= M and col_stride3 > 0 and split_n3 > split_n
     a = LinearArgs(C.sizeof(LinearArgs), code, epilogue, _p(x), K, _p(row_src), _p(row_scale), _p(w), _p(w2), K, _p(bias),
                    M, N, K, _p(group_off), n_groups, N * K if n_groups else 0, _p(y), y.shape[-1] if ldy is None else ldy, out_f32,
                    _p(row_dst), _p(base), N, _p(col_scale), split_n, _p(y2), _p(row_off2), head_dim2, head_stride2,
-                   int(act), int(act_split), int(act2), float(act_param))
+                   split_n3, _p(y3), _p(row_off3), col_stride3, int(act), int(act_split), int(act2), float(act_param))
     check(load().pcb_linear(C.byref(a), _stream()), "pcb_linear")
 
 
@@ -382,22 +388,25 @@ def moe_mix(pair_out: torch.Tensor, expert: torch.Tensor, weight: torch.Tensor, 
     check(load().pcb_moe_mix(_p(pair_out), _p(expert), _p(weight), _p(h), _code(h), n_real, _p(y), n_rows, W, top, _stream()), "pcb_moe_mix")
 
 
-def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, kcache: torch.Tensor, v_offset: int, slot_stride: int,
-                 head_stride: int, row_stride: int, H: int, Hkv: int, dim: int, vdim: int, scale: float, out: torch.Tensor, *,
+def attn_softmax(q: torch.Tensor, ldq: int, tiles: torch.Tensor, n_tiles: int, kcache: torch.Tensor, k_strides, vcache: torch.Tensor,
+                 v_offset: int, v_strides, v_cols: bool, H: int, Hkv: int, dim: int, vdim: int, scale: float, out: torch.Tensor, *,
                  q_scale: Optional[torch.Tensor] = None, window: int = 0, gate: Optional[torch.Tensor] = None, ldg: int = 0,
                  n_splits: int = 1, part: Optional[torch.Tensor] = None) -> None:
-    """``q``: E rows (row stride ``ldq``, head h at column h * dim); ``kcache``: the plane that holds the keys, the values
-    ``v_offset`` elements behind them; ``gate``: E rows of stride ``ldg``; ``out`` E [rows, H * vdim].  ``n_splits`` > 1: each
-    (tile, head) runs as that many workgroups over runs of the keys, merged by a second launch; ``part``: fp32 scratch of
-    ``attn_softmax_part(rows, H, n_splits, vdim)`` floats."""
+    """``q``: E rows (row stride ``ldq``, head h at column h * dim); ``kcache`` with ``k_strides`` = (slot, head, row) strides in
+    elements; the values start ``v_offset`` elements into ``vcache`` (which may be the same plane) with ``v_strides`` = (slot, head,
+    row) strides, or (slot, head, column) strides when ``v_cols`` (a cache kept column by column, columns readable in multiples of
+    32 keys); ``gate``: E rows of stride ``ldg``; ``out`` E [rows, H * vdim].  ``n_splits`` > 1: each (tile, head) runs as that many
+    workgroups over runs of the keys, merged by a second launch; ``part``: fp32 scratch of ``attn_softmax_part(rows, H, n_splits,
+    vdim)`` floats."""
     _want(tiles, torch.int32, "attn_softmax tiles"); _want(q_scale, torch.float32, "attn_softmax q_scale")
-    assert q.dtype == kcache.dtype == out.dtype and out.is_contiguous() and kcache.is_cuda and q.is_cuda
+    assert q.dtype == kcache.dtype == vcache.dtype == out.dtype and out.is_contiguous() and kcache.is_cuda and vcache.is_cuda and q.is_cuda
     assert tiles.numel() >= 4 * n_tiles and out.shape[-1] == H * vdim and ldq >= H * dim
     assert gate is None or (gate.dtype == q.dtype and ldg >= H * vdim)
-    es = kcache.element_size()
+    es = vcache.element_size()
     a = AttnSoftmaxArgs(C.sizeof(AttnSoftmaxArgs), _code(q), _p(q), ldq, _p(q_scale), _p(tiles), n_tiles, _p(kcache),
-                        kcache.data_ptr() + v_offset * es, slot_stride, head_stride, row_stride, H, Hkv, dim, vdim, float(scale),
-                        int(window), _p(gate), ldg, _p(out), out.shape[-1], int(n_splits), _p(part))
+                        vcache.data_ptr() + v_offset * es, int(k_strides[0]), int(k_strides[1]), int(k_strides[2]), int(v_strides[0]),
+                        int(v_strides[1]), int(v_strides[2]), int(v_cols), H, Hkv, dim, vdim, float(scale), int(window), _p(gate), ldg,
+                        _p(out), out.shape[-1], int(n_splits), _p(part))
     if n_splits > 1:
         _want(part, torch.float32, "attn_softmax part")
         assert part.numel() >= attn_softmax_part(out.shape[0], H, n_splits, vdim)

@@ -6,8 +6,9 @@ products on the bf16 matrix cores, fp32 accumulation) or float32 (everything in 
 another, each request continuing from what its slot of the ``SlotArena`` holds.  Nothing is padded, and a row reads nothing but
 its own slot, so a request's numbers do not depend on the rest of the step.
 
-What a slot holds differs by layer: an attention layer keeps keys and values (one plane, a row = the key then the value of a
-position; a layer that borrows another layer's keys and values keeps nothing), a lightning layer one fp32 matrix per head, a
+What a slot holds differs by layer: an attention layer keeps keys (row by row) and values (column by column, so that the matrix
+cores' value operand -- eight positions of one column -- is read with wide loads; a layer that borrows another layer's keys and
+values keeps nothing), a lightning layer one fp32 matrix per head, a
 mamba layer its fp32 scan state and the last inputs of its convolution.
 
 There are S residual streams X_1..X_S (fp32, all equal to the embedding rows at first).  Sublayer by sublayer (f = mixer or
@@ -19,7 +20,7 @@ feed-forward, with its own in / mix / out weights and Dynamic-Tanh norm):
 
     lightning   q | k | v | g = silu, silu, silu, sigmoid of ONE projection; per head S <- decay S + k v^T, o = S^T q
                 (pcb_decay_attn); y = Wo (rms(o) gain * g)                           (pcb_gated_norm)
-    attention   q | g | k,v of ONE projection whose k,v columns land in the slot's cache rows; softmax(temp(pos) scale q.k) v,
+    attention   q | g | k | v of ONE projection whose k and v columns land in the slot's cache; softmax(temp(pos) scale q.k) v,
                 times sigmoid(g) in the attention kernel's store (pcb_attn_softmax); y = Wo (.)
     mamba1      x | z = Win h; x = silu(conv(x)) (pcb_causal_conv); dt_low | B | C = Wx x; dt = softplus(Wdt dt_low + b);
                 S <- exp(dt A) S + dt x B, y = (S C + D x) silu(z) (pcb_selective_scan); y = Wo (.)
@@ -95,11 +96,7 @@ class DibizenHIP(SlotModel):
             elif l.kind == "attention":
                 if max(l.dim, l.vdim) > 256:
                     raise ValueError(f"layer {i}: attention heads take up to 256 columns (got {l.dim} / {l.vdim})")
-                parts = [e(m + "q"), e(m + "g")]
-                if l.kv_from < 0:
-                    k = e(m + "k").view(l.kv_heads, l.dim, self.W)
-                    v = e(m + "v").view(l.kv_heads, l.vdim, self.W)
-                    parts.append(torch.cat([k, v], dim=1).reshape(l.kv_heads * (l.dim + l.vdim), self.W))
+                parts = [e(m + "q"), e(m + "g")] + ([e(m + "k"), e(m + "v")] if l.kv_from < 0 else [])
                 ent.update(w_in=torch.cat(parts, dim=0).contiguous(), wo=e(m + "o"))
             else:
                 if l.state > 256 or l.conv > 16:
@@ -123,23 +120,25 @@ class DibizenHIP(SlotModel):
         self.max_graphs = 16
         # which (coef, every) pairs the attention layers' query temperatures use: one fp32 factor per row and pair
         self._temps = sorted({(l.qt_coef, l.qt_every) for l in shape.layers if l.kind == "attention" and l.qt_every})
-        self._sigs = sorted({(l.kv_heads, l.dim + l.vdim) for l in shape.layers if l.kind == "attention" and l.kv_from < 0})
+        # cache offsets of a row, one table per distinct (heads, columns) of the key planes and of the value planes
+        self._sigs = sorted({(l.kv_heads, l.dim) for l in shape.layers if l.kind == "attention" and l.kv_from < 0})
+        self._vsigs = sorted({(l.kv_heads, l.vdim) for l in shape.layers if l.kind == "attention" and l.kv_from < 0})
 
     # ---- cache and state -------------------------------------------------------------------------------------------------------
     def new_arena(self, slots: int, cap: int) -> SlotArena:
-        dims, states = [], []
+        dims, cols, states = [], [], []
         f32 = torch.float32
         for l in self.config.layers:
-            if l.kind == "attention":
-                dims.append((l.kv_heads, l.dim + l.vdim) if l.kv_from < 0 else (0, 0))
-                states.append([])
-            elif l.kind == "lightning":
-                dims.append((0, 0))
+            own = l.kind == "attention" and l.kv_from < 0
+            dims.append((l.kv_heads, l.dim) if own else (0, 0))          # keys row by row
+            cols.append((l.kv_heads, l.vdim) if own else (0, 0))         # values column by column
+            if l.kind == "lightning":
                 states.append([((l.heads, l.dim, l.vdim), f32)])
-            else:
-                dims.append((0, 0))
+            elif l.kind == "mamba1":
                 states.append([((l.inner, l.state), f32), ((l.conv - 1, l.inner), self.dtype)])
-        return SlotArena(dims, slots, cap, self.device, self.dtype, states=states)
+            else:
+                states.append([])
+        return SlotArena(dims, slots, cap, self.device, self.dtype, states=states, col_dims=cols)
 
     def kv_bytes_per_token(self) -> int:
         es = 2 if self.dtype == torch.bfloat16 else 4
@@ -209,7 +208,8 @@ class DibizenHIP(SlotModel):
             seg_n = seg_a[:, 2].astype(np.float32)
         temps = np.stack([1.0 + coef * np.log(np.floor((row_pos + 1) / every) + 1.0) for coef, every in self._temps]).astype(np.float32) \
             if self._temps else np.zeros((0, T), np.float32)
-        offs = np.stack([row_slot * (g * arena.cap * d) + row_pos * d for g, d in self._sigs]) if self._sigs else np.zeros((0, T), np.int64)
+        offs = np.stack([row_slot * (g * arena.cap * d) + row_pos * d for g, d in self._sigs] +
+                        [row_slot * (g * d * arena.cap) + row_pos for g, d in self._vsigs]) if self._sigs else np.zeros((0, T), np.int64)
         # one block: int32 tables, then fp32 temperatures, then int64 cache offsets
         parts32 = [ids, row_pos.astype(np.int32), meta.reshape(-1), reqs.reshape(-1), tiles.reshape(-1), want_rows, seg_a.reshape(-1),
                    seg_c.reshape(-1), chains.reshape(-1)]
@@ -246,7 +246,8 @@ class DibizenHIP(SlotModel):
         out["temps"] = f32[:nf].view(len(self._temps), T)
         out["seg_n"] = f32[nf:nf + ns]
         out["n_seg"], out["n_chains"] = ns, d["n_chains"]
-        out["offs"] = dblob[d["o64"]:d["o64"] + len(self._sigs) * T * 8].view(torch.int64).view(len(self._sigs), T)
+        no = len(self._sigs) + len(self._vsigs)
+        out["offs"] = dblob[d["o64"]:d["o64"] + no * T * 8].view(torch.int64).view(no, T)
         return out
 
     def _run(self, arena, dblob, d, logits, num_layers=None, return_streams=False):
@@ -322,13 +323,16 @@ class DibizenHIP(SlotModel):
         B.linear(on, lw["wo"], y, M=T)
 
     def _attention(self, arena, i, l, lw, h, y, tb, T, n_tiles):
-        HD, HV, dv = l.heads * l.dim, l.heads * l.vdim, l.dim + l.vdim
+        HD, HV, GD = l.heads * l.dim, l.heads * l.vdim, l.kv_heads * l.dim
         src = i if l.kv_from < 0 else l.kv_from
-        plane = arena.planes[src]
+        plane, vplane = arena.planes[src], arena.col_planes[src]
         qg = self._mat("mix_in", T, HD + HV, self.dtype)
         if l.kv_from < 0:
+            # one projection: q | g stay rows, the k columns go to the slot's key rows, the v columns to its value columns
             B.linear(h, lw["w_in"], qg, M=T, act_split=HD, act2=B.ACT_SIGMOID, split_n=HD + HV, y2=plane,
-                     row_off2=tb["offs"][self._sigs.index((l.kv_heads, dv))], head_dim2=dv, head_stride2=arena.head_stride(src))
+                     row_off2=tb["offs"][self._sigs.index((l.kv_heads, l.dim))], head_dim2=l.dim, head_stride2=arena.head_stride(src),
+                     split_n3=HD + HV + GD, y3=vplane, row_off3=tb["offs"][len(self._sigs) + self._vsigs.index((l.kv_heads, l.vdim))],
+                     col_stride3=arena.cap)
         else:
             B.linear(h, lw["w_in"], qg, M=T, act_split=HD, act2=B.ACT_SIGMOID)
         att = self._mat("mix_out", T, HV, self.dtype)
@@ -336,8 +340,9 @@ class DibizenHIP(SlotModel):
         # few (tile, head) pairs cannot fill the chip: each is cut into runs of its keys (steps of few rows over long caches)
         splits = 1 if n_tiles * l.heads >= 512 or arena.cap <= 256 else max(1, min(16, 1024 // (n_tiles * l.heads), arena.cap // 128))
         part = self._scratch("attn_part", B.attn_softmax_part(T, l.heads, splits, l.vdim), torch.float32) if splits > 1 else None
-        B.attn_softmax(qg, HD + HV, tb["tiles"], n_tiles, plane, l.dim, arena.slot_stride(src), arena.head_stride(src), dv, l.heads,
-                       l.kv_heads, l.dim, l.vdim, l.scale, att, q_scale=temp, gate=qg[:, HD:], ldg=HD + HV, n_splits=splits, part=part)
+        B.attn_softmax(qg, HD + HV, tb["tiles"], n_tiles, plane, (arena.slot_stride(src), arena.head_stride(src), l.dim), vplane, 0,
+                       (arena.col_slot_stride(src), arena.col_head_stride(src), arena.cap), True, l.heads, l.kv_heads, l.dim, l.vdim,
+                       l.scale, att, q_scale=temp, gate=qg[:, HD:], ldg=HD + HV, n_splits=splits, part=part)
         B.linear(att, lw["wo"], y, M=T)
 
     def _mamba(self, arena, i, l, lw, h, y, tb, T, R):

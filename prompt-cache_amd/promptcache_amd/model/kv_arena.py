@@ -293,8 +293,13 @@ class SlotArena:
     ``self.states[layer]``.  A state is not cleared when its slot changes hands: whoever reads it treats a request that starts
     at position 0 as starting from zero."""
 
-    def __init__(self, layer_dims, slots: int, cap: int, device, dtype=torch.bfloat16, states=None):
+    def __init__(self, layer_dims, slots: int, cap: int, device, dtype=torch.bfloat16, states=None, col_dims=None):
         self.layer_dims = [(int(g), int(d)) for g, d in layer_dims]
+        # a second plane per layer kept COLUMN by column, ``[slots][heads][columns][cap]`` (values whose readers want a run of
+        # positions of one column contiguous); with any of these, cap is kept a multiple of 32 so that a reader may fetch whole
+        # blocks of 32 positions
+        self.col_dims = [(int(g), int(d)) for g, d in (col_dims or [(0, 0)] * len(self.layer_dims))]
+        self.col_planes: List[torch.Tensor] = []
         self.state_specs = [[(tuple(int(v) for v in shp), dt) for shp, dt in (per or [])] for per in (states or [[]] * len(self.layer_dims))]
         self.states: List[List[torch.Tensor]] = [[] for _ in self.state_specs]
         self.device, self.dtype = torch.device(device), dtype
@@ -315,7 +320,14 @@ class SlotArena:
         return self.cap * self.layer_dims[layer][1]
 
     def bytes_per_token(self) -> int:
-        return sum(g * d for g, d in self.layer_dims) * torch.empty(0, dtype=self.dtype).element_size()
+        return sum(g * d for g, d in self.layer_dims + self.col_dims) * torch.empty(0, dtype=self.dtype).element_size()
+
+    def col_slot_stride(self, layer: int) -> int:
+        g, d = self.col_dims[layer]
+        return g * d * self.cap
+
+    def col_head_stride(self, layer: int) -> int:
+        return self.col_dims[layer][1] * self.cap
 
     def state_bytes_per_slot(self) -> int:
         n = 0
@@ -330,13 +342,19 @@ class SlotArena:
     def reserve(self, slots: int, cap: int) -> None:
         """At least ``slots`` slots of at least ``cap`` positions each."""
         slots, cap = max(slots, self.slots), max(cap, self.cap)
+        if any(g * d for g, d in self.col_dims):
+            cap = -(-cap // 32) * 32
         if slots == self.slots and cap == self.cap:
             return
         new = [torch.empty((slots, g, cap, d), device=self.device, dtype=self.dtype) for g, d in self.layer_dims]
         keep = max([self.lengths[s] for s in self._live], default=0)
+        new_cols = [torch.empty((slots, g, d, cap), device=self.device, dtype=self.dtype) for g, d in self.col_dims]
         if keep:
             for old, nw in zip(self.planes, new):
                 nw[:self.slots, :, :keep].copy_(old[:, :, :keep])
+            for old, nw in zip(self.col_planes, new_cols):
+                nw[:self.slots, :, :, :keep].copy_(old[:, :, :, :keep])
+        self.col_planes = new_cols
         if slots != self.slots:
             grown = [[torch.zeros((slots, *shp), device=self.device, dtype=dt) for shp, dt in per] for per in self.state_specs]
             for old_l, new_l in zip(self.states, grown):

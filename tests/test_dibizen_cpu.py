@@ -125,6 +125,17 @@ def test_slot_arena_states_follow_their_slots():
     assert ar.alloc() == a and ar.lengths[a] == 0   # handed out again; whoever takes it starts at position 0
 
 
+def test_slot_arena_column_planes_keep_their_columns_when_rows_grow():
+    ar = SlotArena([(2, 4)], 1, 5, "cpu", torch.float32, col_dims=[(2, 3)])
+    assert ar.cap == 32 and tuple(ar.col_planes[0].shape) == (1, 2, 3, 32) and ar.col_head_stride(0) == 96 and ar.col_slot_stride(0) == 192
+    a = ar.alloc()
+    ar.col_planes[0][a, :, :, :7] = torch.arange(7.0)
+    ar.lengths[a] = 7
+    ar.room_for(a, 40)                               # rows grow: every column keeps its first 7 positions
+    assert ar.cap == 64 and torch.equal(ar.col_planes[0][a, 1, 2, :7], torch.arange(7.0))
+    assert ar.bytes_per_token() == (2 * 4 + 2 * 3) * 4
+
+
 # ---- the blocks library's argument structures --------------------------------------------------------------------------------------
 def test_blocks_struct_layouts_match_the_header(tmp_path):
     from promptcache_amd import _blocks

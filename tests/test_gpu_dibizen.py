@@ -134,6 +134,28 @@ def test_linear_activations_and_their_split(dtype, M):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M", [2, 37, 140])
+def test_linear_three_destinations(dtype, M):
+    # columns [0, 20) stay rows, [20, 32) go to a row-wise cache (2 heads of 6), [32, 52) to a column-wise cache (2 heads of 10)
+    N, K, cap = 52, 44, 64
+    x, w = rnd(M, K, dtype=dtype, seed=1), rnd(N, K, dtype=dtype, seed=2, scale=0.3)
+    z = x.to(F64) @ w.to(F64).T
+    slot = torch.arange(M) % 3
+    pos = torch.arange(M) // 3
+    kc = torch.zeros((3, 2, cap, 6), dtype=dtype, device=DEV)
+    vc = torch.zeros((3, 2, 10, cap), dtype=dtype, device=DEV)
+    off2 = (slot * (2 * cap * 6) + pos * 6).to(torch.int64).to(DEV)
+    off3 = (slot * (2 * 10 * cap) + pos).to(torch.int64).to(DEV)
+    y = torch.empty((M, 20), dtype=dtype, device=DEV)
+    B().linear(x, w, y, M=M, act=B().ACT_SIGMOID, split_n=20, y2=kc, row_off2=off2, head_dim2=6, head_stride2=cap * 6, split_n3=32,
+               y3=vc, row_off3=off3, col_stride3=cap)
+    assert rel(y, torch.sigmoid(z[:, :20])) < tol(dtype, 1e-5, 4e-3)
+    got_k = kc[slot, :, pos].reshape(M, 12)
+    got_v = vc[slot, :, :, pos].reshape(M, 20)
+    assert rel(got_k, z[:, 20:32]) < tol(dtype, 1e-5, 4e-3) and rel(got_v, z[:, 32:]) < tol(dtype, 1e-5, 4e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("S", [1, 2, 5])
 def test_hyper_norm_write_read_gather_and_embedding(dtype, S):
     T, Wd = 9, 70
@@ -194,10 +216,11 @@ def test_router_select_and_moe_mix(E, top, groups, keep):
     assert rel(y, (w.unsqueeze(-1) * src).sum(dim=1)) < 1e-6
 
 
-def attention_case(dtype, H, G, D, Dv, lens, news, seed=0, boost=None, splits=1):
-    """``lens[b]`` keys of request b are in the cache (its slot b of a plane with interleaved key | value rows), the last
-    ``news[b]`` of them belong to this step's queries.  Returns (kernel output, oracle output)."""
-    cap, Bn = max(lens) + 3, len(lens)
+def attention_case(dtype, H, G, D, Dv, lens, news, seed=0, boost=None, splits=1, v_cols=False):
+    """``lens[b]`` keys of request b are in the cache (its slot b), the last ``news[b]`` of them belong to this step's queries.
+    The cache is one plane with interleaved key | value rows, or (``v_cols``) key rows plus a value plane kept column by column.
+    Returns (kernel output, oracle output)."""
+    cap, Bn = -(-(max(lens) + 3) // 32) * 32, len(lens)
     plane = rnd(Bn, G, cap, D + Dv, dtype=dtype, seed=seed + 1)
     T = sum(news)
     q = rnd(T, H * D + 5, dtype=dtype, seed=seed + 2)
@@ -215,8 +238,16 @@ def attention_case(dtype, H, G, D, Dv, lens, news, seed=0, boost=None, splits=1)
         row0 += m
     out = torch.empty((T, H * Dv), dtype=dtype, device=DEV)
     part = torch.empty(B().attn_softmax_part(T, H, splits, Dv), dtype=torch.float32, device=DEV) if splits > 1 else None
-    B().attn_softmax(q, H * D + 5, dev_i32(tiles), len(tiles), plane, D, G * cap * (D + Dv), cap * (D + Dv), D + Dv, H, G, D, Dv, 0.3, out,
-                     q_scale=qs, gate=gate, ldg=H * Dv, n_splits=splits, part=part)
+    rows = (G * cap * (D + Dv), cap * (D + Dv), D + Dv)
+    if v_cols:
+        vt = plane[..., D:].permute(0, 1, 3, 2).contiguous()                     # [slots, G, Dv, cap]
+        for b, n in enumerate(lens):
+            vt[b, :, :, n:] = float("nan")                                       # what lies past a request's keys need not be numbers
+        B().attn_softmax(q, H * D + 5, dev_i32(tiles), len(tiles), plane, rows, vt, 0, (G * Dv * cap, Dv * cap, cap), True, H, G, D, Dv,
+                         0.3, out, q_scale=qs, gate=gate, ldg=H * Dv, n_splits=splits, part=part)
+    else:
+        B().attn_softmax(q, H * D + 5, dev_i32(tiles), len(tiles), plane, rows, plane, D, rows, False, H, G, D, Dv, 0.3, out,
+                         q_scale=qs, gate=gate, ldg=H * Dv, n_splits=splits, part=part)
     want, row0 = [], 0
     for b, (n, m) in enumerate(zip(lens, news)):
         qq = q[row0:row0 + m, :H * D].to(F64).cpu().view(m, H, D) * qs[row0:row0 + m].to(F64).cpu().view(m, 1, 1)
@@ -228,18 +259,20 @@ def attention_case(dtype, H, G, D, Dv, lens, news, seed=0, boost=None, splits=1)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("v_cols", [False, True])
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 56, 48), (3, 1, 10, 6), (8, 8, 32, 64), (2, 1, 128, 72), (2, 2, 160, 136), (5, 5, 64, 20)])
-def test_softmax_attention_alone(dtype, H, G, D, Dv):
+def test_softmax_attention_alone(dtype, H, G, D, Dv, v_cols):
     # prompts that end inside a 32-key block and a 16-query tile, a one-token step far into a cache, a first token
-    got, want = attention_case(dtype, H, G, D, Dv, lens=[45, 131, 1, 32, 33], news=[45, 1, 1, 17, 2], seed=H)
+    got, want = attention_case(dtype, H, G, D, Dv, lens=[45, 131, 1, 32, 33], news=[45, 1, 1, 17, 2], seed=H, v_cols=v_cols)
     assert rel(got, want) < tol(dtype, 1e-5, 1.5e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("splits", [2, 5, 16])
-def test_softmax_attention_in_runs_of_the_keys(dtype, splits):
+@pytest.mark.parametrize("splits,v_cols", [(2, False), (5, True), (16, True), (16, False)])
+def test_softmax_attention_in_runs_of_the_keys(dtype, splits, v_cols):
     # more runs than some requests have key blocks: empty runs must drop out of the merge
-    got, want = attention_case(dtype, 4, 2, 48, 40, lens=[45, 700, 1, 32, 33, 257], news=[45, 1, 1, 17, 2, 1], seed=splits, splits=splits)
+    got, want = attention_case(dtype, 4, 2, 48, 40, lens=[45, 700, 1, 32, 33, 257], news=[45, 1, 1, 17, 2, 1], seed=splits, splits=splits,
+                               v_cols=v_cols)
     assert rel(got, want) < tol(dtype, 1e-5, 1.5e-2)
 
 
@@ -247,7 +280,8 @@ def test_softmax_attention_in_runs_of_the_keys(dtype, splits):
 @pytest.mark.parametrize("key,splits", [(0, 1), (31, 1), (32, 4), (127, 1), (128, 4), (299, 1), (299, 7)])
 def test_softmax_attention_finds_a_far_key(dtype, key, splits):
     # the last query's score for ONE key of 300 is raised far above the rest: its head's output must be that key's value
-    got, want = attention_case(dtype, 2, 1, 40, 24, lens=[300, 300], news=[1, 20], seed=3, boost=(1, key, 1, 60.0), splits=splits)
+    got, want = attention_case(dtype, 2, 1, 40, 24, lens=[300, 300], news=[1, 20], seed=3, boost=(1, key, 1, 60.0), splits=splits,
+                               v_cols=key % 2 == 1)
     assert rel(got, want) < tol(dtype, 1e-5, 1.5e-2)
     assert rel(got[-1, 24:], want[-1, 24:]) < tol(dtype, 1e-5, 1.5e-2)
 
