@@ -29,11 +29,14 @@ struct PFrag<float> {
 };
 
 __device__ __forceinline__ void make_p(PFrag<bf16_t>& f, const float (&p)[8]) {
+    // hi = the upper 16 bits of p as they stand, lo = the rest, cut to 16 bits: hi + lo carries 16 bits of p's mantissa (p is a
+    // finite non-negative weight, so no rounding carry or NaN needs care)
     uint32_t h[8], l[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        h[e] = bf16_bits(p[e]);
-        l[e] = bf16_bits(p[e] - __uint_as_float(h[e] << 16));
+        const uint32_t u = __float_as_uint(p[e]);
+        h[e] = u >> 16;
+        l[e] = __float_as_uint(p[e] - __uint_as_float(u & 0xffff0000u)) >> 16;
     }
     f.hi.v = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
     f.lo.v = u32x4{l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16)};
@@ -104,7 +107,9 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
     __shared__ float red_o[AW - 1][VB * 256];
     __shared__ float red_ml[AW - 1][2][16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, c = lane & 15;
-    const int32_t* tile = a.tiles + 4 * blockIdx.x;
+    // (the launch walks the tiles from the last to the first: within a request later tiles see more keys, and the long ones should
+    // not be the ones that start last)
+    const int32_t* tile = a.tiles + 4 * (gridDim.x - 1 - blockIdx.x);
     const int slot = tile[0], pos0 = tile[1], rows = tile[2], row0 = tile[3];
     const int h = blockIdx.y, hk = h / (a.H / a.Hkv);
     const int dim = a.dim, vdim = a.vdim;
@@ -121,7 +126,8 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
     Frag<E> qf[KSQ];
 #pragma unroll
     for (int ks = 0; ks < KSQ; ++ks) qf[ks] = load_frag(qp + 32 * ks, g, dim - 32 * ks, qvec);
-    const float sc = a.scale * (a.q_scale ? a.q_scale[qrow] : 1.0f);
+    // scores are kept in units of ln 2 (the factor log2(e) rides on the scale), so that every exponential is one v_exp_f32
+    const float sc = a.scale * (a.q_scale ? a.q_scale[qrow] : 1.0f) * 1.44269504088896f;
     const float NEG = -__builtin_inff();
 
     float m = NEG, l = 0.0f;
@@ -136,21 +142,55 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
         kb_lo += (int)blockIdx.z * per;
         kb_hi = kb_lo + per - 1 < kb_hi ? kb_lo + per - 1 : kb_hi;
     }
-    for (int kb = kb_lo + wave; kb <= kb_hi; kb += AW) {
-        float s[8];
+    // the key operands of a block are requested one block ahead (where the registers allow it), so that their latency hides behind
+    // the block in work
+    constexpr bool PREK = sizeof(E) == 2 ? KSQ <= 4 : KSQ <= 2;
+    Frag<E> kn[PREK ? 2 : 1][PREK ? KSQ : 1];
+    auto fetch_k = [&](int kb) {
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
             int j = kb * 32 + kt * 16 + c;                  // this lane's key row of the K operand
             j = j > last ? last : j;
             const E* kp = K + (int64_t)j * a.row_stride;
+#pragma unroll
+            for (int ks = 0; ks < KSQ; ++ks) kn[PREK ? kt : 0][PREK ? ks : 0] = load_frag(kp + 32 * ks, g, dim - 32 * ks, kvec);
+        }
+    };
+    if (PREK && kb_lo + wave <= kb_hi) fetch_k(kb_lo + wave);
+    for (int kb = kb_lo + wave; kb <= kb_hi; kb += AW) {
+        float s[8];
+        Frag<E> kc[PREK ? 2 : 1][PREK ? KSQ : 1];
+        if (PREK) {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int ks = 0; ks < KSQ; ++ks) kc[PREK ? kt : 0][PREK ? ks : 0] = kn[PREK ? kt : 0][PREK ? ks : 0];
+            if (kb + AW <= kb_hi) fetch_k(kb + AW);
+        }
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            int j = kb * 32 + kt * 16 + c;
+            j = j > last ? last : j;
+            const E* kp = K + (int64_t)j * a.row_stride;
             f4 acc = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < KSQ; ++ks) acc = mma(load_frag(kp + 32 * ks, g, dim - 32 * ks, kvec), qf[ks], acc);
+            for (int ks = 0; ks < KSQ; ++ks)
+                acc = mma(PREK ? kc[PREK ? kt : 0][PREK ? ks : 0] : load_frag(kp + 32 * ks, g, dim - 32 * ks, kvec), qf[ks], acc);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = kb * 32 + kt * 16 + 4 * g + r;
                 const bool seen = key <= qpos && (a.window <= 0 || qpos - key < a.window);
                 s[kt * 4 + r] = seen ? acc[r] * sc : NEG;
+            }
+        }
+        // the value operands are requested before the softmax arithmetic (column-wise cache: two wide loads per 16 columns)
+        const int v_valid = last + 1 - kb * 32;             // keys of this block that exist
+        Frag<E> vfs[VB];
+        if (a.v_cols) {
+#pragma unroll
+            for (int vb = 0; vb < VB; ++vb) {
+                const int col = vb * 16 + c;
+                if (vb * 16 < vdim) vfs[vb] = load_v_cols(V + (int64_t)(col < vdim ? col : 0) * a.v_stride + kb * 32, g, col < vdim, v_valid);
             }
         }
         float bm = s[0];
@@ -160,11 +200,11 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
         bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
         const float m_new = fmaxf(m, bm);
         const float m_use = m_new == NEG ? 0.0f : m_new;
-        const float alpha = expf(m - m_use);                // (m = -inf: 0)
+        const float alpha = __builtin_amdgcn_exp2f(m - m_use);      // (m = -inf: 0)
         float p[8], psum = 0.0f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            p[e] = expf(s[e] - m_use);
+            p[e] = __builtin_amdgcn_exp2f(s[e] - m_use);
             psum += p[e];
         }
         l = l * alpha + psum;
@@ -178,13 +218,11 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
             key = key > last ? last : key;
             vrows[e] = V + (int64_t)key * a.v_stride;
         }
-        const int v_valid = last + 1 - kb * 32;             // keys of this block that exist
 #pragma unroll
         for (int vb = 0; vb < VB; ++vb) {
             if (vb * 16 >= vdim) break;
             const int col = vb * 16 + c;
-            const Frag<E> vf = a.v_cols ? load_v_cols(V + (int64_t)(col < vdim ? col : 0) * a.v_stride + kb * 32, g, col < vdim, v_valid)
-                                        : load_v(vrows, col, col < vdim);
+            const Frag<E> vf = a.v_cols ? vfs[vb] : load_v(vrows, col, col < vdim);
             f4 t = o[vb];
 #pragma unroll
             for (int r = 0; r < 4; ++r) t[r] *= alpha;
@@ -212,7 +250,7 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
 #pragma unroll
     for (int w = 0; w < AW - 1; ++w) mm = fmaxf(mm, red_ml[w][0][c]);
     const float m_use = mm == NEG ? 0.0f : mm;
-    float f0 = expf(m - m_use);
+    float f0 = __builtin_amdgcn_exp2f(m - m_use);
     float lt = l * f0;
 #pragma unroll
     for (int vb = 0; vb < VB; ++vb)
@@ -220,7 +258,7 @@ __global__ __launch_bounds__(64 * AW) void attn_softmax_kernel(pcb_attn_softmax_
         for (int r = 0; r < 4; ++r) o[vb][r] *= f0;
 #pragma unroll
     for (int w = 0; w < AW - 1; ++w) {
-        const float fw = expf(red_ml[w][0][c] - m_use);
+        const float fw = __builtin_amdgcn_exp2f(red_ml[w][0][c] - m_use);
         lt += red_ml[w][1][c] * fw;
 #pragma unroll
         for (int vb = 0; vb < VB; ++vb)
@@ -271,7 +309,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(pcb_attn_softmax_args a
         const float m_use = mm == NEG ? 0.0f : mm;
         float l = 0.0f, o = 0.0f;
         for (int z = 0; z < Z; ++z) {
-            const float f = expf(pp[z * (vdim + 2) + vdim] - m_use);
+            const float f = __builtin_amdgcn_exp2f(pp[z * (vdim + 2) + vdim] - m_use);      // (maxima are in units of ln 2)
             l += f * pp[z * (vdim + 2) + vdim + 1];
             o += f * pp[z * (vdim + 2) + col];
         }
