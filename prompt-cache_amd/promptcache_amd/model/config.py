@@ -404,7 +404,7 @@ class DibizenShape:
                     raise ValueError(f"layer {i}: top {lay.top} of {total} router outputs with {lay.groups_keep} of {lay.groups} groups")
             layers.append(lay)
         return cls(vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), norm_eps=float((c.get("norm") or {}).get("eps", 1e-5)),
-                   layers=layers, streams=int(c.get("streams", 1)), max_positions=int(c["max_positions"]),
+                   layers=layers, streams=int(c.get("streams", 1)), max_positions=int(c.get("max_positions") or 0),
                    logit_softcap=float(c.get("logit_softcap") or 0.0), name=name)
 
     @classmethod

@@ -433,7 +433,8 @@ def load_dibizen_safetensors(path: str, cfg):
         raise KeyError(f"{path}: tensors missing for this configuration: {missing[:6]}{' ...' if len(missing) > 6 else ''}")
     for k, shp in want.items():
         if k == "pos" and raw[k].dim() == 2 and raw[k].shape[1] == shp[1]:
-            continue                                  # (the table's own length says how many positions there are)
+            cfg.max_positions = int(raw[k].shape[0])  # (the table's own length says how many positions there are)
+            continue
         if tuple(raw[k].shape) != tuple(shp):
             raise ValueError(f"{path}: {k} has shape {tuple(raw[k].shape)}, the configuration implies {tuple(shp)}")
     return {k: raw[k] for k in want}
